@@ -1,0 +1,259 @@
+/*
+ * libxabe_hip: the quantized MoE feed-forward block for one MI355X (gfx950).
+ *
+ * C ABI that a Rust FFI crate binds in place of `xabe_cuda::kernels::moe`.
+ * Each entry point names the reference item it replaces; paths are relative to
+ * the reference tree, "M" = crates/xabe-cuda/src/kernels/moe.rs,
+ * "B" = crates/xabe-engine/src/block/moe.rs, "D" = crates/xabe-engine/src/block/dense_ffn.rs.
+ *
+ * Conventions
+ *   - Every function returns an `xabe_status` (0 = ok).  `xabe_last_error()` gives the
+ *     message of the calling thread's last failure, worded like the reference's
+ *     `MoeError` / `MoeBlockError` Display impls.
+ *   - Device memory is passed as a raw pointer plus an element count, the way the
+ *     reference passes `&CudaSlice<T>`; lengths are checked where the reference checks them.
+ *   - `stream` is a `hipStream_t` passed as `void*` (NULL = the default stream).
+ *   - Every launch is asynchronous on `stream`, sized from the geometry only, and reads the
+ *     live token count from the device scalar `valid_tokens` (M:34-41): the sequence can be
+ *     captured into a hipGraph.  No entry point allocates except the `_new` / `_upload` ones.
+ *   - One kernels+buffers pair per pass shape per thread; calls on one buffer set must not overlap.
+ */
+#ifndef XABE_HIP_H
+#define XABE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes: MoeError (M:4602-4637) and MoeBlockError (B:494-547) ---- */
+typedef enum xabe_status {
+  XABE_OK = 0,
+  XABE_ERR_COMPILE = 1,               /* MoeError::Compile: the code object failed to load on this device */
+  XABE_ERR_DRIVER = 2,                /* MoeError::Driver: a HIP runtime call failed */
+  XABE_ERR_MMA = 3,                   /* MoeError::Mma: the matrix-core path rejected its operands */
+  XABE_ERR_UNSUPPORTED_GEOMETRY = 4,  /* MoeError::UnsupportedGeometry { geometry, reason } */
+  XABE_ERR_RAGGED_WEIGHTS = 5,        /* MoeError::RaggedWeights { which, bytes, block_bytes } */
+  XABE_ERR_WRONG_ELEMENT_COUNT = 6,   /* MoeError::WrongElementCount { which, expected, found } */
+  XABE_ERR_TOO_MANY_TOKENS = 7,       /* MoeError::TooManyTokens { tokens, max_tokens } */
+  XABE_ERR_SHARED_ONLY_BUFFERS = 8,   /* MoeError::SharedOnlyBuffers { entry } */
+  XABE_ERR_BUFFER_LENGTH = 9,         /* MoeBlockError::BufferLength { what, expected, found } */
+  XABE_ERR_INVALID_ARGUMENT = 10,     /* a NULL handle or pointer (the Rust API rules this out by type) */
+  XABE_ERR_UNSUPPORTED_QUANT = 11,    /* MoeBlockError::UnsupportedExpertType: Q4_0/Q4_K/Q5_K have no kernel here */
+  XABE_ERR_FFN_KIND_MISMATCH = 12     /* MoeBlockError::FfnKindMismatch */
+} xabe_status;
+
+const char* xabe_last_error(void);
+const char* xabe_status_name(int status);
+/* Library version and the architecture the code object was built for ("gfx950"). */
+const char* xabe_version(void);
+
+/* ---- MoeGeometry (M:4523-4598) ---- */
+typedef struct xabe_moe_geometry {
+  size_t num_experts;
+  size_t experts_per_token;
+  size_t hidden;
+  size_t intermediate;
+  size_t block_size;
+  size_t max_tokens;
+} xabe_moe_geometry;
+
+/* MoeGeometry::qwen3_6 (M:4544-4553) */
+xabe_moe_geometry xabe_moe_geometry_qwen3_6(size_t block_size, size_t max_tokens);
+size_t xabe_moe_geometry_max_flat_pairs(const xabe_moe_geometry* g);         /* M:4556-4558 */
+size_t xabe_moe_geometry_sorted_capacity(const xabe_moe_geometry* g);        /* M:4575-4584 */
+size_t xabe_moe_geometry_expert_block_capacity(const xabe_moe_geometry* g);  /* M:4587-4589 */
+size_t xabe_moe_geometry_stack_elements(const xabe_moe_geometry* g);         /* M:4595-4597 */
+/* crates/xabe-engine/src/forward.rs:163-165: 32 up to 1152 tokens, else 64 */
+size_t xabe_moe_block_size_for(size_t tokens);
+
+/* ---- ExpertQuant (M:298-401), QuantTensor (M:448-464), to_device_layout (M:410-444) ---- */
+typedef enum xabe_expert_quant {
+  XABE_QUANT_Q6K = 0,
+  XABE_QUANT_Q8_0 = 1,
+  XABE_QUANT_Q4_0 = 2, /* community formats: recognised, rejected with XABE_ERR_UNSUPPORTED_QUANT */
+  XABE_QUANT_Q4K = 3,
+  XABE_QUANT_Q5K = 4
+} xabe_expert_quant;
+
+size_t xabe_expert_quant_block_elements(int quant);   /* M:353-360 */
+size_t xabe_expert_quant_file_block_bytes(int quant); /* M:366-374 */
+/* M:388-400.  Equal to file_block_bytes for every format: the kernels stream the 210-byte
+ * Q6_K superblock as the file stores it, so there is no 224-byte device stride. */
+size_t xabe_expert_quant_block_bytes(int quant);
+int xabe_expert_quant_is_community(int quant);        /* M:348-350 */
+
+/* A quantized stack resident on the device.  `bytes` is a device pointer to `len` bytes. */
+typedef struct xabe_quant_tensor {
+  const void* bytes;
+  size_t len;
+  int quant;
+} xabe_quant_tensor;
+
+/* M:410-444.  The identity copy: `out` (host, `len` bytes) receives `bytes` unchanged and
+ * `*out_len = len`.  Kept so callers that route every upload through the hook keep working. */
+int xabe_to_device_layout(int quant, const uint8_t* bytes, size_t len, uint8_t* out, size_t* out_len);
+
+/* ---- MoeKernels (M:5033-5458) ---- */
+typedef struct xabe_moe_kernels xabe_moe_kernels;
+typedef struct xabe_moe_buffers xabe_moe_buffers;
+
+typedef enum xabe_buffer_scope { XABE_SCOPE_ROUTED = 0, XABE_SCOPE_SHARED_ONLY = 1 } xabe_buffer_scope; /* M:4698-4705 */
+
+/* MoeKernels::new (M:5038-5330): validates the geometry (same rules, same reasons) and
+ * loads the gfx950 code object on the current device. */
+int xabe_moe_kernels_new(const xabe_moe_geometry* geometry, xabe_moe_kernels** out);
+void xabe_moe_kernels_free(xabe_moe_kernels* k);
+int xabe_moe_kernels_geometry(const xabe_moe_kernels* k, xabe_moe_geometry* out); /* M:5333 */
+/* M:5416-5418: force the matrix-core (MFMA) regime off; prefill widths then take the fp32 kernels. */
+int xabe_moe_kernels_disable_tensor_cores(xabe_moe_kernels* k);
+int xabe_moe_kernels_tensor_cores_enabled(const xabe_moe_kernels* k);             /* M:5456-5458 */
+/* M:5432-5434: no community-format kernels exist here; `on != 0` is accepted and recorded only. */
+int xabe_moe_kernels_force_community(xabe_moe_kernels* k, int on);
+/* M:5450-5452: pin the fp32 decode kernels at any width so rows equal plain decode bit for bit. */
+int xabe_moe_kernels_set_exact_decode_regime(xabe_moe_kernels* k, int on);
+
+/* MoeKernels::buffers (M:5338-5340) / shared_only_buffers (M:5354-5360) */
+int xabe_moe_buffers_new(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers** out);
+int xabe_moe_shared_only_buffers_new(const xabe_moe_kernels* k, void* stream, int mma, xabe_moe_buffers** out);
+void xabe_moe_buffers_free(xabe_moe_buffers* b);
+
+/* MoeBuffers accessors (M:4768-4864): device pointer + element count. */
+int xabe_moe_buffers_scope(const xabe_moe_buffers* b);
+int32_t* xabe_moe_buffers_topk_ids(const xabe_moe_buffers* b, size_t* len);
+float* xabe_moe_buffers_topk_weights(const xabe_moe_buffers* b, size_t* len);
+int32_t* xabe_moe_buffers_sorted_token_ids(const xabe_moe_buffers* b, size_t* len);
+int32_t* xabe_moe_buffers_expert_ids(const xabe_moe_buffers* b, size_t* len);
+int32_t* xabe_moe_buffers_bucket_live(const xabe_moe_buffers* b, size_t* len);
+int32_t* xabe_moe_buffers_num_tokens_post_pad(const xabe_moe_buffers* b, size_t* len);
+int32_t* xabe_moe_buffers_valid_tokens(const xabe_moe_buffers* b, size_t* len);
+float* xabe_moe_buffers_partial(const xabe_moe_buffers* b, size_t* len);
+float* xabe_moe_buffers_shared_inter(const xabe_moe_buffers* b, size_t* len);
+size_t xabe_moe_buffers_bytes(const xabe_moe_buffers* b);
+
+/* MoeKernels::set_valid_tokens (M:5473-5491): one 4-byte host-to-device write, skipped when unchanged. */
+int xabe_moe_set_valid_tokens(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, size_t tokens);
+
+/* MoeKernels::route (M:5567-5609): softmax, top-k (probability descending, lower index on ties),
+ * renormalise.  `logits` is [max_tokens][num_experts]. */
+int xabe_moe_route(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, const float* logits, size_t logits_len);
+/* MoeKernels::build_dispatch (M:5623-5714) */
+int xabe_moe_build_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b);
+/* MoeKernels::route_and_dispatch (M:5498-5558): the dispatch tables are skipped when the flat
+ * per-pair kernels will run (max_tokens <= 4, or the exact decode regime). */
+int xabe_moe_route_and_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, const float* logits,
+                                size_t logits_len);
+
+/* MoeKernels::grouped_forward_partial (M:5727-6170): leaves partial[(t*K+k)*hidden ..] = w_{t,k} * y. */
+int xabe_moe_grouped_forward_partial(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b,
+                                     xabe_quant_tensor gate, xabe_quant_tensor up, xabe_quant_tensor down,
+                                     const float* hidden_states, size_t hidden_states_len);
+/* MoeKernels::grouped_forward_partial_with_shared (M:6190-6335).  `*fused` = 1 when the shared
+ * expert rode the routed launches, 0 (nothing launched) when the pass is not covered. */
+int xabe_moe_grouped_forward_partial_with_shared(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b,
+                                                 xabe_quant_tensor gate, xabe_quant_tensor up, xabe_quant_tensor down,
+                                                 xabe_quant_tensor shared_gate, xabe_quant_tensor shared_up,
+                                                 xabe_quant_tensor shared_down, const float* hidden_states,
+                                                 size_t hidden_states_len, float* out, size_t out_len, int* fused);
+/* MoeKernels::grouped_forward (M:6345-6376): partial + the ascending-k sum (`moe_reduce`, M:4049-4065). */
+int xabe_moe_grouped_forward(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                             xabe_quant_tensor up, xabe_quant_tensor down, const float* hidden_states,
+                             size_t hidden_states_len, float* out, size_t out_len);
+/* MoeKernels::shared_expert (M:6488-6714): expert_mlp on every live token, ungated.  Also the dense
+ * sibling's MLP (D:34-43): widths come from the geometry, stacks are single-expert. */
+int xabe_moe_shared_expert(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                           xabe_quant_tensor up, xabe_quant_tensor down, const float* hidden_states,
+                           size_t hidden_states_len, float* out, size_t out_len);
+/* MoeKernels::shared_expert_mma (M:6389-6476) with SharedExpertInt8::repack (M:4896-4938) folded in:
+ * the matrix-core path reads the quantized stacks directly, so there is nothing to repack. */
+int xabe_moe_shared_expert_mma(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                               xabe_quant_tensor up, xabe_quant_tensor down, const float* hidden_states,
+                               size_t hidden_states_len, float* out, size_t out_len);
+
+/* ---- kernels the engine compiled for itself through NVRTC; here they are library entry points ---- */
+/* LayerOpsKernels::rms_norm (crates/xabe-cuda/src/kernels/layer_ops.rs:777-805): every row, 1/sqrtf. */
+int xabe_rms_norm(void* stream, const float* x, size_t x_len, const float* weight, size_t weight_len, float* out,
+                  size_t out_len, size_t rows, size_t width, float eps);
+/* moe_block_router_logits (B:301-382, launch B:1150-1184).  `router` is f32 [E][H], or Q8_0 bytes
+ * dequantised in-kernel as q*d when `router_quant` is XABE_QUANT_Q8_0 (pass -1 for f32). */
+int xabe_moe_router_logits(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b, const void* router,
+                           size_t router_len, int router_quant, const float* normed, size_t normed_len, float* logits,
+                           size_t logits_len);
+/* moe_block_gate_and_combine (B:424-483, launch B:1297-1326) */
+int xabe_moe_gate_and_combine(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b,
+                              const float* shared_gate_inp, const float* normed, const float* shexp,
+                              const float* residual, float* gate, float* routed, float* ffn_out, float* l_out);
+/* dense_ffn_add_residual (D:1149-1175): l_out = ffn_out + residual on live rows. */
+int xabe_dense_ffn_add_residual(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b,
+                                const float* ffn_out, const float* residual, float* l_out);
+/* Adds `bias[e]` to every live row of `logits` (a harness hook: skewed-routing workloads add a
+ * per-expert bias between the router GEMV and `route`; no counterpart in the reference). */
+int xabe_moe_add_logit_bias(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b, const float* bias,
+                            float* logits);
+/* Standalone dequantisation, bit-identical to the CPU reference
+ * (crates/xabe-cuda/src/kernels/dequant.rs:19-27). `out` holds blocks*block_elements floats. */
+int xabe_dequantize(void* stream, int quant, const void* bytes, size_t len, float* out, size_t out_len);
+
+/* ---- MoeBlock / MoeLayerWeights (B:634-1330) and DenseFfnBlock (D:1047-1178): block sequencing ---- */
+typedef struct xabe_moe_block xabe_moe_block;
+
+/* Device-resident tensors of one layer (B:634-658).  The router may be f32 or Q8_0. */
+typedef struct xabe_moe_layer_weights {
+  const float* post_norm;       /* [hidden] */
+  const void* router;           /* [num_experts][hidden] */
+  int router_quant;             /* -1 = f32, XABE_QUANT_Q8_0 = quantized */
+  xabe_quant_tensor gate_exps, up_exps, down_exps;
+  const float* shared_gate_inp; /* [hidden] */
+  xabe_quant_tensor shared_gate, shared_up, shared_down;
+} xabe_moe_layer_weights;
+
+/* MoeBlock::new (B:948-977): kernels, buffers and the normed/logits/routed/shexp/gate scratch. */
+int xabe_moe_block_new(const xabe_moe_geometry* geometry, float eps, void* stream, xabe_moe_block** out);
+void xabe_moe_block_free(xabe_moe_block* blk);
+int xabe_moe_block_publish_tokens(xabe_moe_block* blk, void* stream, size_t tokens); /* B:1081-1089 */
+/* MoeBlock::forward (B:1091-1329).  residual / ffn_out / l_out are [max_tokens][hidden];
+ * `logit_bias` (may be NULL) is added to the router logits before routing. */
+int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
+                           size_t residual_len, size_t tokens, const float* logit_bias, float* ffn_out,
+                           size_t ffn_out_len, float* l_out, size_t l_out_len);
+int xabe_moe_block_disable_tensor_cores(xabe_moe_block* blk);            /* B:987-989 */
+int xabe_moe_block_set_exact_decode_regime(xabe_moe_block* blk, int on); /* B:1003-1005 */
+int xabe_moe_block_tensor_cores_enabled(const xabe_moe_block* blk);      /* B:1008-1010 */
+/* Read-back accessors (B:1023-1060): device pointer + element count. */
+const float* xabe_moe_block_normed(const xabe_moe_block* blk, size_t* len);
+const float* xabe_moe_block_router_logits(const xabe_moe_block* blk, size_t* len);
+const float* xabe_moe_block_routed(const xabe_moe_block* blk, size_t* len);
+const float* xabe_moe_block_shared_ungated(const xabe_moe_block* blk, size_t* len);
+const float* xabe_moe_block_shared_gate(const xabe_moe_block* blk, size_t* len);
+xabe_moe_buffers* xabe_moe_block_buffers(const xabe_moe_block* blk);
+xabe_moe_kernels* xabe_moe_block_kernels(const xabe_moe_block* blk);
+
+typedef struct xabe_dense_ffn_block xabe_dense_ffn_block;
+typedef struct xabe_dense_ffn_layer_weights {
+  const float* post_norm; /* [hidden] */
+  xabe_quant_tensor gate, up, down;
+} xabe_dense_ffn_layer_weights;
+/* DenseFfnBlock::new / forward (D:1047-1178): shared-only buffers, rms_norm -> shared_expert -> residual add. */
+int xabe_dense_ffn_block_new(size_t hidden, size_t intermediate, size_t max_tokens, float eps, void* stream,
+                             xabe_dense_ffn_block** out);
+void xabe_dense_ffn_block_free(xabe_dense_ffn_block* blk);
+int xabe_dense_ffn_block_forward(xabe_dense_ffn_block* blk, void* stream, const xabe_dense_ffn_layer_weights* w,
+                                 const float* residual, size_t residual_len, size_t tokens, float* ffn_out,
+                                 size_t ffn_out_len, float* l_out, size_t l_out_len);
+int xabe_dense_ffn_block_disable_tensor_cores(xabe_dense_ffn_block* blk);
+const float* xabe_dense_ffn_block_normed(const xabe_dense_ffn_block* blk, size_t* len);
+
+/* ---- synthetic stacks for benches (the role of crates/xabe-cuda/src/bin/bench_moe.rs:140-334) ----
+ * Fills device memory with seeded values: element i belongs to chunk i/256, chunk c draws from
+ * xorshift64*(splitmix64(seed + c*0x9E3779B97F4A7C15)); each value is sigma times an Irwin-Hall(12)
+ * normal approximation computed in integer arithmetic; quantized with the reference's own amax
+ * quantizers (crates/xabe-kernels/src/quant.rs:75-88, :495-567). */
+int xabe_synth_normal_f32(void* stream, uint64_t seed, size_t n, float sigma, float* out);
+int xabe_synth_quant(void* stream, int quant, uint64_t seed, size_t n_elements, float sigma, void* out, size_t out_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XABE_HIP_H */

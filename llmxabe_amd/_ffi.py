@@ -1,0 +1,131 @@
+"""ctypes loader for libxabe_hip.so (the C ABI declared in include/xabe_hip.h).
+
+There is no fallback: if the library is missing or a symbol does not resolve the import
+fails, and every wrapper raises on a non-zero status."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libxabe_hip.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "xabe_hip.h")
+
+sz = C.c_size_t
+vp = C.c_void_p
+
+
+class Geometry(C.Structure):
+    _fields_ = [("num_experts", sz), ("experts_per_token", sz), ("hidden", sz), ("intermediate", sz),
+                ("block_size", sz), ("max_tokens", sz)]
+
+
+class QuantTensorC(C.Structure):
+    _fields_ = [("bytes", vp), ("len", sz), ("quant", C.c_int)]
+
+
+class MoeLayerWeightsC(C.Structure):
+    _fields_ = [("post_norm", vp), ("router", vp), ("router_quant", C.c_int),
+                ("gate_exps", QuantTensorC), ("up_exps", QuantTensorC), ("down_exps", QuantTensorC),
+                ("shared_gate_inp", vp),
+                ("shared_gate", QuantTensorC), ("shared_up", QuantTensorC), ("shared_down", QuantTensorC)]
+
+
+class DenseLayerWeightsC(C.Structure):
+    _fields_ = [("post_norm", vp), ("gate", QuantTensorC), ("up", QuantTensorC), ("down", QuantTensorC)]
+
+
+_SIGNATURES = {
+    "xabe_last_error": (C.c_char_p, []),
+    "xabe_status_name": (C.c_char_p, [C.c_int]),
+    "xabe_version": (C.c_char_p, []),
+    "xabe_moe_geometry_qwen3_6": (Geometry, [sz, sz]),
+    "xabe_moe_geometry_max_flat_pairs": (sz, [C.POINTER(Geometry)]),
+    "xabe_moe_geometry_sorted_capacity": (sz, [C.POINTER(Geometry)]),
+    "xabe_moe_geometry_expert_block_capacity": (sz, [C.POINTER(Geometry)]),
+    "xabe_moe_geometry_stack_elements": (sz, [C.POINTER(Geometry)]),
+    "xabe_moe_block_size_for": (sz, [sz]),
+    "xabe_expert_quant_block_elements": (sz, [C.c_int]),
+    "xabe_expert_quant_file_block_bytes": (sz, [C.c_int]),
+    "xabe_expert_quant_block_bytes": (sz, [C.c_int]),
+    "xabe_expert_quant_is_community": (C.c_int, [C.c_int]),
+    "xabe_to_device_layout": (C.c_int, [C.c_int, vp, sz, vp, C.POINTER(sz)]),
+    "xabe_moe_kernels_new": (C.c_int, [C.POINTER(Geometry), C.POINTER(vp)]),
+    "xabe_moe_kernels_free": (None, [vp]),
+    "xabe_moe_kernels_geometry": (C.c_int, [vp, C.POINTER(Geometry)]),
+    "xabe_moe_kernels_disable_tensor_cores": (C.c_int, [vp]),
+    "xabe_moe_kernels_tensor_cores_enabled": (C.c_int, [vp]),
+    "xabe_moe_kernels_force_community": (C.c_int, [vp, C.c_int]),
+    "xabe_moe_kernels_set_exact_decode_regime": (C.c_int, [vp, C.c_int]),
+    "xabe_moe_buffers_new": (C.c_int, [vp, vp, C.POINTER(vp)]),
+    "xabe_moe_shared_only_buffers_new": (C.c_int, [vp, vp, C.c_int, C.POINTER(vp)]),
+    "xabe_moe_buffers_free": (None, [vp]),
+    "xabe_moe_buffers_scope": (C.c_int, [vp]),
+    "xabe_moe_buffers_topk_ids": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_topk_weights": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_sorted_token_ids": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_expert_ids": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_bucket_live": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_num_tokens_post_pad": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_valid_tokens": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_partial": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_shared_inter": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_buffers_bytes": (sz, [vp]),
+    "xabe_moe_set_valid_tokens": (C.c_int, [vp, vp, vp, sz]),
+    "xabe_moe_route": (C.c_int, [vp, vp, vp, vp, sz]),
+    "xabe_moe_build_dispatch": (C.c_int, [vp, vp, vp]),
+    "xabe_moe_route_and_dispatch": (C.c_int, [vp, vp, vp, vp, sz]),
+    "xabe_moe_grouped_forward_partial": (C.c_int, [vp, vp, vp, QuantTensorC, QuantTensorC, QuantTensorC, vp, sz]),
+    "xabe_moe_grouped_forward_partial_with_shared": (C.c_int, [vp, vp, vp] + [QuantTensorC] * 6 + [vp, sz, vp, sz, C.POINTER(C.c_int)]),
+    "xabe_moe_grouped_forward": (C.c_int, [vp, vp, vp, QuantTensorC, QuantTensorC, QuantTensorC, vp, sz, vp, sz]),
+    "xabe_moe_shared_expert": (C.c_int, [vp, vp, vp, QuantTensorC, QuantTensorC, QuantTensorC, vp, sz, vp, sz]),
+    "xabe_moe_shared_expert_mma": (C.c_int, [vp, vp, vp, QuantTensorC, QuantTensorC, QuantTensorC, vp, sz, vp, sz]),
+    "xabe_rms_norm": (C.c_int, [vp, vp, sz, vp, sz, vp, sz, sz, sz, C.c_float]),
+    "xabe_moe_router_logits": (C.c_int, [vp, vp, vp, vp, sz, C.c_int, vp, sz, vp, sz]),
+    "xabe_moe_gate_and_combine": (C.c_int, [vp] * 11),
+    "xabe_dense_ffn_add_residual": (C.c_int, [vp] * 6),
+    "xabe_moe_add_logit_bias": (C.c_int, [vp] * 5),
+    "xabe_dequantize": (C.c_int, [vp, C.c_int, vp, sz, vp, sz]),
+    "xabe_moe_block_new": (C.c_int, [C.POINTER(Geometry), C.c_float, vp, C.POINTER(vp)]),
+    "xabe_moe_block_free": (None, [vp]),
+    "xabe_moe_block_publish_tokens": (C.c_int, [vp, vp, sz]),
+    "xabe_moe_block_forward": (C.c_int, [vp, vp, C.POINTER(MoeLayerWeightsC), vp, sz, sz, vp, vp, sz, vp, sz]),
+    "xabe_moe_block_disable_tensor_cores": (C.c_int, [vp]),
+    "xabe_moe_block_set_exact_decode_regime": (C.c_int, [vp, C.c_int]),
+    "xabe_moe_block_tensor_cores_enabled": (C.c_int, [vp]),
+    "xabe_moe_block_normed": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_block_router_logits": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_block_routed": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_block_shared_ungated": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_block_shared_gate": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_block_buffers": (vp, [vp]),
+    "xabe_moe_block_kernels": (vp, [vp]),
+    "xabe_dense_ffn_block_new": (C.c_int, [sz, sz, sz, C.c_float, vp, C.POINTER(vp)]),
+    "xabe_dense_ffn_block_free": (None, [vp]),
+    "xabe_dense_ffn_block_forward": (C.c_int, [vp, vp, C.POINTER(DenseLayerWeightsC), vp, sz, sz, vp, sz, vp, sz]),
+    "xabe_dense_ffn_block_disable_tensor_cores": (C.c_int, [vp]),
+    "xabe_dense_ffn_block_normed": (vp, [vp, C.POINTER(sz)]),
+    "xabe_synth_normal_f32": (C.c_int, [vp, C.c_uint64, sz, C.c_float, vp]),
+    "xabe_synth_quant": (C.c_int, [vp, C.c_int, C.c_uint64, sz, C.c_float, vp, sz]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """The loaded library.  Raises ImportError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `make -C llmxabe_amd/csrc` (or __graft_entry__.build()). "
+                "There is no CPU fallback.")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(L, name)  # AttributeError if the symbol is not exported
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib

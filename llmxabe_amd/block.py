@@ -1,0 +1,118 @@
+"""Block-level mirrors of `MoeBlock` / `MoeLayerWeights` (crates/xabe-engine/src/block/moe.rs:634-1330)
+and `DenseFfnBlock` (crates/xabe-engine/src/block/dense_ffn.rs).  The sequencing itself lives in the
+library (csrc/block.hip); these classes hold the handles and the device tensors."""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _ffi
+from ._ffi import DenseLayerWeightsC, MoeLayerWeightsC
+from .moe import ExpertQuant, MoeBuffers, MoeGeometry, QuantTensor, _ptr, _stream, _wrap, check
+
+DEFAULT_RMS_EPS = 1e-6  # block/moe.rs:179
+
+
+@dataclass
+class MoeLayerWeights:
+    """Device tensors of one layer (block/moe.rs:634-658).  `router` is f32 [E][H] when
+    `router_quant` is None, else Q8_0 bytes."""
+    post_norm: torch.Tensor
+    router: torch.Tensor
+    router_quant: Optional[ExpertQuant]
+    gate_exps: QuantTensor
+    up_exps: QuantTensor
+    down_exps: QuantTensor
+    shared_gate_inp: torch.Tensor
+    shared_gate: QuantTensor
+    shared_up: QuantTensor
+    shared_down: QuantTensor
+
+    def _c(self) -> MoeLayerWeightsC:
+        return MoeLayerWeightsC(_ptr(self.post_norm), _ptr(self.router),
+                                -1 if self.router_quant is None else int(self.router_quant),
+                                self.gate_exps._c(), self.up_exps._c(), self.down_exps._c(),
+                                _ptr(self.shared_gate_inp), self.shared_gate._c(), self.shared_up._c(),
+                                self.shared_down._c())
+
+
+class MoeBlock:
+    def __init__(self, geometry: MoeGeometry, eps: float = DEFAULT_RMS_EPS):
+        h = C.c_void_p()
+        check(_ffi.lib().xabe_moe_block_new(C.byref(geometry._c()), eps, _stream(), C.byref(h)))
+        self._h = h.value
+        self._geometry = geometry
+        self._eps = eps
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            _ffi.lib().xabe_moe_block_free(self._h)
+            self._h = None
+
+    def geometry(self) -> MoeGeometry: return self._geometry
+    def eps(self) -> float: return self._eps
+    def disable_tensor_cores(self): check(_ffi.lib().xabe_moe_block_disable_tensor_cores(self._h))
+    def set_exact_decode_regime(self, on: bool): check(_ffi.lib().xabe_moe_block_set_exact_decode_regime(self._h, int(on)))
+    def tensor_cores_enabled(self) -> bool: return bool(_ffi.lib().xabe_moe_block_tensor_cores_enabled(self._h))
+
+    def publish_tokens(self, tokens: int):
+        check(_ffi.lib().xabe_moe_block_publish_tokens(self._h, _stream(), tokens))
+
+    def forward(self, w: MoeLayerWeights, residual, tokens: int, ffn_out, l_out, logit_bias=None):
+        cw = w._c()
+        check(_ffi.lib().xabe_moe_block_forward(self._h, _stream(), C.byref(cw), _ptr(residual), residual.numel(), tokens,
+                                                _ptr(logit_bias), _ptr(ffn_out), ffn_out.numel(), _ptr(l_out),
+                                                l_out.numel()))
+
+    def _view(self, name: str) -> torch.Tensor:
+        n = C.c_size_t(0)
+        p = getattr(_ffi.lib(), "xabe_moe_block_" + name)(self._h, C.byref(n))
+        return _wrap(p, n.value, torch.float32)
+
+    def normed(self): return self._view("normed")
+    def router_logits(self): return self._view("router_logits")
+    def routed(self): return self._view("routed")
+    def shared_ungated(self): return self._view("shared_ungated")
+    def shared_gate(self): return self._view("shared_gate")
+
+    def buffers(self) -> MoeBuffers:
+        return MoeBuffers(_ffi.lib().xabe_moe_block_buffers(self._h), owner=False)
+
+
+@dataclass
+class DenseFfnLayerWeights:
+    post_norm: torch.Tensor
+    gate: QuantTensor
+    up: QuantTensor
+    down: QuantTensor
+
+    def _c(self) -> DenseLayerWeightsC:
+        return DenseLayerWeightsC(_ptr(self.post_norm), self.gate._c(), self.up._c(), self.down._c())
+
+
+class DenseFfnBlock:
+    def __init__(self, hidden: int, intermediate: int, max_tokens: int, eps: float = DEFAULT_RMS_EPS):
+        h = C.c_void_p()
+        check(_ffi.lib().xabe_dense_ffn_block_new(hidden, intermediate, max_tokens, eps, _stream(), C.byref(h)))
+        self._h = h.value
+        self.hidden, self.intermediate, self.max_tokens = hidden, intermediate, max_tokens
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            _ffi.lib().xabe_dense_ffn_block_free(self._h)
+            self._h = None
+
+    def disable_tensor_cores(self): check(_ffi.lib().xabe_dense_ffn_block_disable_tensor_cores(self._h))
+
+    def forward(self, w: DenseFfnLayerWeights, residual, tokens: int, ffn_out, l_out):
+        cw = w._c()
+        check(_ffi.lib().xabe_dense_ffn_block_forward(self._h, _stream(), C.byref(cw), _ptr(residual), residual.numel(),
+                                                      tokens, _ptr(ffn_out), ffn_out.numel(), _ptr(l_out), l_out.numel()))
+
+    def normed(self) -> torch.Tensor:
+        n = C.c_size_t(0)
+        p = _ffi.lib().xabe_dense_ffn_block_normed(self._h, C.byref(n))
+        return _wrap(p, n.value, torch.float32)

@@ -1,0 +1,214 @@
+// Block sequencing: the host-side mirror of `MoeBlock::forward`
+// (crates/xabe-engine/src/block/moe.rs:1091-1329) and `DenseFfnBlock::forward`
+// (crates/xabe-engine/src/block/dense_ffn.rs:1047-1178), over the C ABI above it.
+#include <string.h>
+
+#include "host_common.h"
+
+using namespace xabe;
+
+struct xabe_moe_block {
+  xabe_moe_kernels* moe;
+  xabe_moe_buffers* buffers;
+  xabe_moe_geometry g;
+  float eps;
+  float *normed, *logits, *routed, *shexp, *gate;
+  size_t n_act, n_logits;
+};
+
+static int block_alloc(float** p, size_t n, hipStream_t s) {
+  XABE_HIP_TRY(hipMalloc(reinterpret_cast<void**>(p), n * sizeof(float)));
+  XABE_HIP_TRY(hipMemsetAsync(*p, 0, n * sizeof(float), s));
+  return XABE_OK;
+}
+
+int xabe_moe_block_new(const xabe_moe_geometry* geometry, float eps, void* stream, xabe_moe_block** out) {
+  if (!geometry || !out) return set_error(XABE_ERR_INVALID_ARGUMENT, "MoeBlock::new: null pointer");
+  xabe_moe_block* blk = new xabe_moe_block();
+  memset(blk, 0, sizeof(*blk));
+  blk->g = *geometry;
+  blk->eps = eps;
+  int st = xabe_moe_kernels_new(geometry, &blk->moe);
+  if (st == XABE_OK) st = xabe_moe_buffers_new(blk->moe, stream, &blk->buffers);
+  blk->n_act = geometry->max_tokens * geometry->hidden;
+  blk->n_logits = geometry->max_tokens * geometry->num_experts;
+  hipStream_t s = as_stream(stream);
+  if (st == XABE_OK) st = block_alloc(&blk->normed, blk->n_act, s);
+  if (st == XABE_OK) st = block_alloc(&blk->logits, blk->n_logits, s);
+  if (st == XABE_OK) st = block_alloc(&blk->routed, blk->n_act, s);
+  if (st == XABE_OK) st = block_alloc(&blk->shexp, blk->n_act, s);
+  if (st == XABE_OK) st = block_alloc(&blk->gate, geometry->max_tokens, s);
+  if (st != XABE_OK) {
+    xabe_moe_block_free(blk);
+    return st;
+  }
+  *out = blk;
+  return XABE_OK;
+}
+
+void xabe_moe_block_free(xabe_moe_block* blk) {
+  if (!blk) return;
+  float* ptrs[] = {blk->normed, blk->logits, blk->routed, blk->shexp, blk->gate};
+  for (float* p : ptrs)
+    if (p) (void)hipFree(p);
+  xabe_moe_buffers_free(blk->buffers);
+  xabe_moe_kernels_free(blk->moe);
+  delete blk;
+}
+
+int xabe_moe_block_publish_tokens(xabe_moe_block* blk, void* stream, size_t tokens) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "publish_tokens: null handle");
+  return xabe_moe_set_valid_tokens(blk->moe, stream, blk->buffers, tokens);
+}
+
+static int blk_check_len(const char* what, size_t expected, size_t found) {
+  if (expected != found) return set_error(XABE_ERR_BUFFER_LENGTH, "%s holds %zu elements, expected %zu", what, found, expected);
+  return XABE_OK;
+}
+
+int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
+                           size_t residual_len, size_t tokens, const float* logit_bias, float* ffn_out,
+                           size_t ffn_out_len, float* l_out, size_t l_out_len) {
+  if (!blk || !w || !residual || !ffn_out || !l_out) return set_error(XABE_ERR_INVALID_ARGUMENT, "MoeBlock::forward: null pointer");
+  const xabe_moe_geometry& g = blk->g;
+  if (tokens > g.max_tokens)
+    return set_error(XABE_ERR_TOO_MANY_TOKENS, "%zu tokens exceeds the %zu the block was sized for", tokens, g.max_tokens);
+  XABE_TRY(blk_check_len("residual", blk->n_act, residual_len));
+  XABE_TRY(blk_check_len("ffn_out", blk->n_act, ffn_out_len));
+  XABE_TRY(blk_check_len("l_out", blk->n_act, l_out_len));
+  XABE_TRY(xabe_moe_block_publish_tokens(blk, stream, tokens));
+
+  // 1. post-mixer RMSNorm over every row of the buffer
+  XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
+                         g.hidden, blk->eps));
+  // 2. router logits, (bias,) softmax + top-k + renormalise, dispatch tables
+  const size_t router_len = w->router_quant < 0
+                                ? g.num_experts * g.hidden
+                                : g.num_experts * g.hidden / xabe_expert_quant_block_elements(w->router_quant) *
+                                      xabe_expert_quant_block_bytes(w->router_quant);
+  XABE_TRY(xabe_moe_router_logits(blk->moe, stream, blk->buffers, w->router, router_len, w->router_quant, blk->normed,
+                                  blk->n_act, blk->logits, blk->n_logits));
+  if (logit_bias) XABE_TRY(xabe_moe_add_logit_bias(blk->moe, stream, blk->buffers, logit_bias, blk->logits));
+  XABE_TRY(xabe_moe_route_and_dispatch(blk->moe, stream, blk->buffers, blk->logits, blk->n_logits));
+  // 3 + 4. routed experts (stopping at `partial`) and the ungated shared expert
+  int fused = 0;
+  const bool wide = g.max_tokens >= kMfmaMinTokens && xabe_moe_kernels_tensor_cores_enabled(blk->moe);
+  if (!wide)
+    XABE_TRY(xabe_moe_grouped_forward_partial_with_shared(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps,
+                                                          w->down_exps, w->shared_gate, w->shared_up, w->shared_down,
+                                                          blk->normed, blk->n_act, blk->shexp, blk->n_act, &fused));
+  if (!fused) {
+    XABE_TRY(xabe_moe_grouped_forward_partial(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps, w->down_exps,
+                                              blk->normed, blk->n_act));
+    if (wide && mfma_supported(blk->moe, blk->buffers, w->shared_gate.quant, w->shared_up.quant, w->shared_down.quant, false))
+      XABE_TRY(xabe_moe_shared_expert_mma(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
+                                          blk->normed, blk->n_act, blk->shexp, blk->n_act));
+    else
+      XABE_TRY(xabe_moe_shared_expert(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
+                                      blk->normed, blk->n_act, blk->shexp, blk->n_act));
+  }
+  // 5. routed sum, sigmoid gate, combine, residual
+  return xabe_moe_gate_and_combine(blk->moe, stream, blk->buffers, w->shared_gate_inp, blk->normed, blk->shexp, residual,
+                                   blk->gate, blk->routed, ffn_out, l_out);
+}
+
+int xabe_moe_block_disable_tensor_cores(xabe_moe_block* blk) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "disable_tensor_cores: null handle");
+  return xabe_moe_kernels_disable_tensor_cores(blk->moe);
+}
+int xabe_moe_block_set_exact_decode_regime(xabe_moe_block* blk, int on) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_exact_decode_regime: null handle");
+  return xabe_moe_kernels_set_exact_decode_regime(blk->moe, on);
+}
+int xabe_moe_block_tensor_cores_enabled(const xabe_moe_block* blk) {
+  return blk ? xabe_moe_kernels_tensor_cores_enabled(blk->moe) : 0;
+}
+
+#define XABE_BLOCK_ACCESSOR(name, field, count)                                   \
+  const float* xabe_moe_block_##name(const xabe_moe_block* blk, size_t* len) {    \
+    if (!blk) { if (len) *len = 0; return nullptr; }                              \
+    if (len) *len = (count);                                                      \
+    return blk->field;                                                            \
+  }
+XABE_BLOCK_ACCESSOR(normed, normed, blk->n_act)
+XABE_BLOCK_ACCESSOR(router_logits, logits, blk->n_logits)
+XABE_BLOCK_ACCESSOR(routed, routed, blk->n_act)
+XABE_BLOCK_ACCESSOR(shared_ungated, shexp, blk->n_act)
+XABE_BLOCK_ACCESSOR(shared_gate, gate, blk->g.max_tokens)
+xabe_moe_buffers* xabe_moe_block_buffers(const xabe_moe_block* blk) { return blk ? blk->buffers : nullptr; }
+xabe_moe_kernels* xabe_moe_block_kernels(const xabe_moe_block* blk) { return blk ? blk->moe : nullptr; }
+
+// ------------------------------------------------------------------ dense sibling
+struct xabe_dense_ffn_block {
+  xabe_moe_kernels* moe;
+  xabe_moe_buffers* buffers;
+  xabe_moe_geometry g;
+  float eps;
+  float* normed;
+  size_t n_act;
+};
+
+int xabe_dense_ffn_block_new(size_t hidden, size_t intermediate, size_t max_tokens, float eps, void* stream,
+                             xabe_dense_ffn_block** out) {
+  if (!out) return set_error(XABE_ERR_INVALID_ARGUMENT, "DenseFfnBlock::new: null pointer");
+  // DenseFfnBlock::geometry_for: one "expert", no routing (dense_ffn.rs)
+  xabe_moe_geometry g = {1, 1, hidden, intermediate, xabe_moe_block_size_for(max_tokens), max_tokens};
+  xabe_dense_ffn_block* blk = new xabe_dense_ffn_block();
+  memset(blk, 0, sizeof(*blk));
+  blk->g = g;
+  blk->eps = eps;
+  blk->n_act = max_tokens * hidden;
+  int st = xabe_moe_kernels_new(&g, &blk->moe);
+  if (st == XABE_OK) st = xabe_moe_shared_only_buffers_new(blk->moe, stream, 1, &blk->buffers);
+  if (st == XABE_OK) st = block_alloc(&blk->normed, blk->n_act, as_stream(stream));
+  if (st != XABE_OK) {
+    xabe_dense_ffn_block_free(blk);
+    return st;
+  }
+  *out = blk;
+  return XABE_OK;
+}
+
+void xabe_dense_ffn_block_free(xabe_dense_ffn_block* blk) {
+  if (!blk) return;
+  if (blk->normed) (void)hipFree(blk->normed);
+  xabe_moe_buffers_free(blk->buffers);
+  xabe_moe_kernels_free(blk->moe);
+  delete blk;
+}
+
+int xabe_dense_ffn_block_disable_tensor_cores(xabe_dense_ffn_block* blk) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "disable_tensor_cores: null handle");
+  return xabe_moe_kernels_disable_tensor_cores(blk->moe);
+}
+
+const float* xabe_dense_ffn_block_normed(const xabe_dense_ffn_block* blk, size_t* len) {
+  if (!blk) { if (len) *len = 0; return nullptr; }
+  if (len) *len = blk->n_act;
+  return blk->normed;
+}
+
+int xabe_dense_ffn_block_forward(xabe_dense_ffn_block* blk, void* stream, const xabe_dense_ffn_layer_weights* w,
+                                 const float* residual, size_t residual_len, size_t tokens, float* ffn_out,
+                                 size_t ffn_out_len, float* l_out, size_t l_out_len) {
+  if (!blk || !w || !residual || !ffn_out || !l_out)
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "DenseFfnBlock::forward: null pointer");
+  const xabe_moe_geometry& g = blk->g;
+  if (tokens > g.max_tokens)
+    return set_error(XABE_ERR_TOO_MANY_TOKENS, "%zu tokens exceeds the %zu the block was sized for", tokens, g.max_tokens);
+  XABE_TRY(blk_check_len("residual", blk->n_act, residual_len));
+  XABE_TRY(blk_check_len("ffn_out", blk->n_act, ffn_out_len));
+  XABE_TRY(blk_check_len("l_out", blk->n_act, l_out_len));
+  XABE_TRY(xabe_moe_set_valid_tokens(blk->moe, stream, blk->buffers, tokens));
+  XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
+                         g.hidden, blk->eps));
+  const bool wide = g.max_tokens >= kMfmaMinTokens && xabe_moe_kernels_tensor_cores_enabled(blk->moe) &&
+                    mfma_supported(blk->moe, blk->buffers, w->gate.quant, w->up.quant, w->down.quant, false);
+  if (wide)
+    XABE_TRY(xabe_moe_shared_expert_mma(blk->moe, stream, blk->buffers, w->gate, w->up, w->down, blk->normed, blk->n_act,
+                                        ffn_out, blk->n_act));
+  else
+    XABE_TRY(xabe_moe_shared_expert(blk->moe, stream, blk->buffers, w->gate, w->up, w->down, blk->normed, blk->n_act,
+                                    ffn_out, blk->n_act));
+  return xabe_dense_ffn_add_residual(blk->moe, stream, blk->buffers, ffn_out, residual, l_out);
+}

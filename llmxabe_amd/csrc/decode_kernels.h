@@ -1,0 +1,362 @@
+// Decode-regime expert kernels: fp32 accumulation, weights streamed once from HBM
+// in their file layout (210-byte Q6_K superblocks / 34-byte Q8_0 blocks), dequantised
+// in registers.  Replaces the reference's gemv / flat / tiled fp32 families
+// (crates/xabe-cuda/src/kernels/moe.rs:2403-3124, :3425-3725, :4082-4227).
+//
+// One wavefront "step" covers 2048 contraction elements of a row: 8 Q6_K superblocks
+// (1680 B) or 64 Q8_0 blocks (2176 B), 32 elements per lane.  Rows shorter than 2048
+// pack RPS = 2048/K rows into a step; longer rows take KS steps, the last one masked.
+// Activations for the lane's fixed element positions live in registers, so a row costs
+// its own bytes and nothing else.
+//
+// Numerics contract: the value of (row, token) is computed by one fixed sequence of
+// fp32 operations that does not depend on which other tokens are present, so a token
+// decodes to the same bits alone or in a batch (tests/test_gpu_batch_invariance.py).
+#pragma once
+
+#include "device_common.h"
+
+namespace xabe {
+
+constexpr int kWavesPerWg = 4;
+
+template <int QUANT>
+struct Fmt;
+template <>
+struct Fmt<kQ6K> {
+  using Raw = Q6Raw;
+  static constexpr uint32_t kChunkBytes = 8 * kQ6KBytes;
+  static constexpr int kBlockElems = 256;
+  static constexpr int kBlockBytes = kQ6KBytes;
+};
+template <>
+struct Fmt<kQ8_0> {
+  using Raw = Q8Raw;
+  static constexpr uint32_t kChunkBytes = 64 * kQ8Bytes;
+  static constexpr int kBlockElems = 32;
+  static constexpr int kBlockBytes = kQ8Bytes;
+};
+
+template <>
+struct Fmt<kF32> {
+  using Raw = F32Raw;
+  static constexpr uint32_t kChunkBytes = 2048 * 4;
+  static constexpr int kBlockElems = 1;
+  static constexpr int kBlockBytes = 4;
+};
+
+struct LaneGeom {
+  int lane, slot, half, l8;
+  uint32_t lane_off;  // byte offset of the lane's block inside a step's chunk
+};
+
+template <int QUANT>
+__device__ __forceinline__ LaneGeom lane_geom() {
+  LaneGeom g;
+  g.lane = __lane_id();
+  g.slot = g.lane >> 3;
+  g.half = (g.lane >> 2) & 1;
+  g.l8 = g.lane & 3;
+  g.lane_off = QUANT == kQ6K ? (uint32_t)g.slot * kQ6KBytes
+             : QUANT == kQ8_0 ? (uint32_t)g.lane * kQ8Bytes
+                              : (uint32_t)g.lane * 128u;
+  return g;
+}
+
+// Offset, within a row, of the first of the 32 elements this lane covers in step `k`.
+// For Q6_K that is the start of the lane's superblock (positions inside it: q6_pos).
+template <int QUANT, int RPS>
+__device__ __forceinline__ int lane_koff(const LaneGeom& g, int k) {
+  if (QUANT == kQ6K) return ((g.slot % (8 / RPS)) + k * 8) * 256;
+  return ((g.lane % (64 / RPS)) + k * 64) * 32;
+}
+
+template <int QUANT>
+__device__ __forceinline__ void load_x(const float* __restrict__ xrow, int koff, bool active, const LaneGeom& g,
+                                       float (&x)[32], float (&xs)[4]) {
+  if (QUANT == kQ6K) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+      if (active) {
+        const float4* p = reinterpret_cast<const float4*>(xrow + koff + g.half * 128 + j * 32 + g.l8 * 8);
+        a = p[0];
+        b = p[1];
+      }
+      x[j * 8 + 0] = a.x; x[j * 8 + 1] = a.y; x[j * 8 + 2] = a.z; x[j * 8 + 3] = a.w;
+      x[j * 8 + 4] = b.x; x[j * 8 + 5] = b.y; x[j * 8 + 6] = b.z; x[j * 8 + 7] = b.w;
+      float s = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s += x[j * 8 + i];
+      xs[j] = -32.0f * s;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (active) a = reinterpret_cast<const float4*>(xrow + koff)[j];
+      x[j * 4 + 0] = a.x; x[j * 4 + 1] = a.y; x[j * 4 + 2] = a.z; x[j * 4 + 3] = a.w;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xs[j] = 0.0f;
+  }
+}
+
+template <int QUANT>
+__device__ __forceinline__ void raw_zero(typename Fmt<QUANT>::Raw& r);
+template <>
+__device__ __forceinline__ void raw_zero<kQ6K>(Q6Raw& r) {
+  r.qa0 = r.qa1 = r.qb0 = r.qb1 = r.qh0 = r.qh1 = r.sc0 = r.sc1 = r.dh = 0;
+}
+template <>
+__device__ __forceinline__ void raw_zero<kQ8_0>(Q8Raw& r) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r.q[i] = 0;
+  r.dh = 0;
+}
+template <>
+__device__ __forceinline__ void raw_zero<kF32>(F32Raw& r) {
+#pragma unroll
+  for (int i = 0; i < 32; ++i) r.v[i] = 0.0f;
+}
+
+// Loads this lane's block of the step that starts at `chunk` (any 2-byte alignment).
+template <int QUANT>
+__device__ __forceinline__ void load_raw(const uint8_t* chunk, bool active, const LaneGeom& g,
+                                         typename Fmt<QUANT>::Raw& r) {
+  if (!active) {
+    raw_zero<QUANT>(r);
+    return;
+  }
+  const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(chunk) & 3u);
+  const uint8_t* chunk4 = chunk - mis;
+  if constexpr (QUANT == kQ6K) q6_load(chunk4, g.lane_off + mis, g.half, g.l8, r);
+  else if constexpr (QUANT == kQ8_0) q8_load(chunk4, g.lane_off + mis, r);
+  else f32_load(chunk, g.lane_off, r);
+}
+
+template <int QUANT, int TC>
+__device__ __forceinline__ void accum(const typename Fmt<QUANT>::Raw& r, const LaneGeom& g, const float (&x)[TC][32],
+                                      const float (&xs)[TC][4], float (&tot)[TC]) {
+  if constexpr (QUANT == kQ6K) q6_accum<TC>(r, g.l8, x, xs, tot);
+  else if constexpr (QUANT == kQ8_0) q8_accum<TC>(r, x, tot);
+  else f32_accum<TC>(r, x, tot);
+}
+
+// ---------------------------------------------------------------------------------
+// matvec_rows: the body every decode kernel shares.
+//   NM = 2: out[t][row] = silu(gate_row . x_t) * (up_row . x_t)      (gate/up + SwiGLU)
+//   NM = 1: out[t][row] = scale[t] * (w_row . x_t)                    (down / plain GEMV)
+// `w0`/`w1` point at row 0 of the matrix (one expert).  Rows [tile0, tile0+tile_rows)
+// are split over the workgroup's four wavefronts.  KS > 0: steps per row, activations
+// in registers.  KS == 0: steps from K at run time, activations re-read per step.
+// ---------------------------------------------------------------------------------
+template <int QUANT, int KS, int RPS, int TC, int NM>
+__device__ __forceinline__ void matvec_rows(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, int K,
+                                            int n_rows, int tile0, int tile_rows,
+                                            const float* const (&xrow)[TC], float* const (&out)[TC],
+                                            const float (&scale)[TC]) {
+  using F = Fmt<QUANT>;
+  using Raw = typename F::Raw;
+  constexpr int G = 64 / RPS;
+  static_assert(RPS == 1 || KS == 1, "short rows take exactly one step");
+  const LaneGeom g = lane_geom<QUANT>();
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const size_t row_bytes = (size_t)(K / F::kBlockElems) * F::kBlockBytes;
+  const int tile_end = min(tile0 + tile_rows, n_rows);
+
+  if constexpr (KS > 0) {
+    float x[KS][TC][32];
+    float xs[KS][TC][4];
+    bool active[KS];
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      const int koff = lane_koff<QUANT, RPS>(g, k);
+      active[k] = koff < K;
+#pragma unroll
+      for (int t = 0; t < TC; ++t) load_x<QUANT>(xrow[t], koff, active[k], g, x[k][t], xs[k][t]);
+    }
+    auto load_item = [&](int row0, Raw (&r)[NM][KS]) {
+#pragma unroll
+      for (int k = 0; k < KS; ++k) {
+        const size_t off = (size_t)row0 * row_bytes + (size_t)k * F::kChunkBytes;
+        load_raw<QUANT>(w0 + off, active[k], g, r[0][k]);
+        if constexpr (NM == 2) load_raw<QUANT>(w1 + off, active[k], g, r[NM - 1][k]);
+      }
+    };
+    auto finish_item = [&](int row0, const Raw (&r)[NM][KS]) {
+      float tot[NM][TC];
+#pragma unroll
+      for (int m = 0; m < NM; ++m) {
+#pragma unroll
+        for (int t = 0; t < TC; ++t) tot[m][t] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KS; ++k) accum<QUANT, TC>(r[m][k], g, x[k], xs[k], tot[m]);
+#pragma unroll
+        for (int t = 0; t < TC; ++t) tot[m][t] = group_sum<G>(tot[m][t]);
+      }
+      const int row = row0 + g.lane / G;
+      if ((g.lane % G) == 0 && row < n_rows) {
+#pragma unroll
+        for (int t = 0; t < TC; ++t) {
+          const float v = NM == 2 ? silu_f(tot[0][t]) * tot[NM - 1][t] : scale[t] * tot[0][t];
+          out[t][row] = v;
+        }
+      }
+    };
+    int row0 = tile0 + wave * RPS;
+    if constexpr (KS == 1) {
+      // software pipeline: the next item's bytes are in flight while this one is reduced
+      Raw cur[NM][KS], nxt[NM][KS];
+      if (row0 < tile_end) load_item(row0, cur);
+      for (; row0 < tile_end; row0 += kWavesPerWg * RPS) {
+        const int nrow = row0 + kWavesPerWg * RPS;
+        if (nrow < tile_end) load_item(nrow, nxt);
+        finish_item(row0, cur);
+#pragma unroll
+        for (int m = 0; m < NM; ++m) cur[m][0] = nxt[m][0];
+      }
+    } else {
+      for (; row0 < tile_end; row0 += kWavesPerWg * RPS) {
+        Raw cur[NM][KS];
+        load_item(row0, cur);
+        finish_item(row0, cur);
+      }
+    }
+  } else {
+    // long rows: K / 2048 steps (last one masked), activations re-read each step
+    const int steps = (K + kStepElems - 1) / kStepElems;
+    for (int row0 = tile0 + wave; row0 < tile_end; row0 += kWavesPerWg) {
+      float tot[NM][TC];
+#pragma unroll
+      for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int t = 0; t < TC; ++t) tot[m][t] = 0.0f;
+      for (int k = 0; k < steps; ++k) {
+        const int koff = lane_koff<QUANT, 1>(g, k);
+        const bool act = koff < K;
+        float x[TC][32];
+        float xs[TC][4];
+#pragma unroll
+        for (int t = 0; t < TC; ++t) load_x<QUANT>(xrow[t], koff, act, g, x[t], xs[t]);
+        const size_t off = (size_t)row0 * row_bytes + (size_t)k * F::kChunkBytes;
+        Raw r0;
+        load_raw<QUANT>(w0 + off, act, g, r0);
+        accum<QUANT, TC>(r0, g, x, xs, tot[0]);
+        if constexpr (NM == 2) {
+          Raw r1;
+          load_raw<QUANT>(w1 + off, act, g, r1);
+          accum<QUANT, TC>(r1, g, x, xs, tot[NM - 1]);
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int t = 0; t < TC; ++t) tot[m][t] = group_sum<64>(tot[m][t]);
+      if (g.lane == 0) {
+#pragma unroll
+        for (int t = 0; t < TC; ++t) {
+          const float v = NM == 2 ? silu_f(tot[0][t]) * tot[NM - 1][t] : scale[t] * tot[0][t];
+          out[t][row0] = v;
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Kernels.  grid.x tiles the output rows, grid.y enumerates work units; every grid is
+// a function of the geometry, the live token count is read from `valid_tokens`.
+// ---------------------------------------------------------------------------------
+struct ExpertArgs {
+  const uint8_t* w0;         // gate stack (NM=2) or down stack (NM=1)
+  const uint8_t* w1;         // up stack (NM=2) or unused
+  size_t expert_bytes;       // bytes of one expert in a stack (0 for a single-expert stack)
+  const float* x;            // activations: [token][K] (gate/up: normed; down: inter rows)
+  float* out;                // gate/up: inter [unit][n_rows]; down: partial/out [unit][n_rows]
+  const int* valid_tokens;   // device scalar
+  const int* topk_ids;       // [T][top_k]
+  const float* topk_weights; // [T][top_k]
+  const int* sorted_token_ids;
+  const int* expert_ids;
+  int K;                     // contraction length
+  int n_rows;                // output rows per expert
+  int top_k;
+  int block_size;
+  int tile_rows;             // rows per workgroup
+};
+
+// Flat regime (max_tokens <= 4, or the exact decode regime): one work unit per live
+// (token, k) pair read straight from topk_ids; no dispatch table
+// (crates/xabe-cuda/src/kernels/moe.rs:2525-2634, :3066-3124).
+template <int QUANT, int KS, int RPS, int NM>
+__global__ void __launch_bounds__(256) k_expert_flat(ExpertArgs a) {
+  const int p = blockIdx.y;
+  const int valid = *a.valid_tokens;
+  if (p >= valid * a.top_k) return;
+  const int e = a.topk_ids[p];
+  const uint8_t* w0 = a.w0 + (size_t)e * a.expert_bytes;
+  const uint8_t* w1 = NM == 2 ? a.w1 + (size_t)e * a.expert_bytes : nullptr;
+  // gate/up reads the token's activation row; down reads the pair's own inter row
+  const float* const xr[1] = {a.x + (size_t)(NM == 2 ? p / a.top_k : p) * a.K};
+  float* const o[1] = {a.out + (size_t)p * a.n_rows};
+  const float sc[1] = {NM == 2 ? 1.0f : a.topk_weights[p]};
+  matvec_rows<QUANT, KS, RPS, 1, NM>(w0, w1, a.K, a.n_rows, blockIdx.x * a.tile_rows, a.tile_rows, xr, o, sc);
+}
+
+// Dispatch-table regime: one work unit per dispatch block; the block's live slots all
+// belong to one expert, whose rows are streamed once per chunk of two tokens
+// (chunks after the first hit in L2).  gate/up writes inter[slot]; down reads
+// inter[slot] and writes partial[flat].
+template <int QUANT, int KS, int RPS, int NM>
+__global__ void __launch_bounds__(256) k_expert_block(ExpertArgs a) {
+  const int b = blockIdx.y;
+  const int e = a.expert_ids[b];
+  if (e < 0) return;
+  const int valid = *a.valid_tokens;
+  const int sentinel = valid * a.top_k;
+  const uint8_t* w0 = a.w0 + (size_t)e * a.expert_bytes;
+  const uint8_t* w1 = NM == 2 ? a.w1 + (size_t)e * a.expert_bytes : nullptr;
+  const int* slots = a.sorted_token_ids + (size_t)b * a.block_size;
+  for (int i = 0; i < a.block_size; i += 2) {
+    const int f0 = slots[i];
+    if (f0 >= sentinel) break;
+    const int f1 = (i + 1 < a.block_size) ? slots[i + 1] : sentinel;
+    const size_t s0 = (size_t)b * a.block_size + i;
+    if (f1 < sentinel) {
+      const float* const xr[2] = {a.x + (NM == 2 ? (size_t)(f0 / a.top_k) : s0) * a.K,
+                                  a.x + (NM == 2 ? (size_t)(f1 / a.top_k) : s0 + 1) * a.K};
+      float* const o[2] = {a.out + (NM == 2 ? s0 : (size_t)f0) * a.n_rows,
+                           a.out + (NM == 2 ? s0 + 1 : (size_t)f1) * a.n_rows};
+      const float sc[2] = {NM == 2 ? 1.0f : a.topk_weights[f0], NM == 2 ? 1.0f : a.topk_weights[f1]};
+      matvec_rows<QUANT, KS, RPS, 2, NM>(w0, w1, a.K, a.n_rows, blockIdx.x * a.tile_rows, a.tile_rows, xr, o, sc);
+    } else {
+      const float* const xr[1] = {a.x + (NM == 2 ? (size_t)(f0 / a.top_k) : s0) * a.K};
+      float* const o[1] = {a.out + (NM == 2 ? s0 : (size_t)f0) * a.n_rows};
+      const float sc[1] = {NM == 2 ? 1.0f : a.topk_weights[f0]};
+      matvec_rows<QUANT, KS, RPS, 1, NM>(w0, w1, a.K, a.n_rows, blockIdx.x * a.tile_rows, a.tile_rows, xr, o, sc);
+    }
+  }
+}
+
+// Shared expert / dense MLP: every live token, no indirection, no routing weight
+// (crates/xabe-cuda/src/kernels/moe.rs:3425-3725, :4082-4227).  One work unit per chunk of two tokens.
+template <int QUANT, int KS, int RPS, int NM>
+__global__ void __launch_bounds__(256) k_expert_shared(ExpertArgs a) {
+  const int t0 = blockIdx.y * 2;
+  const int valid = *a.valid_tokens;
+  if (t0 >= valid) return;
+  if (t0 + 1 < valid) {
+    const float* const xr[2] = {a.x + (size_t)t0 * a.K, a.x + (size_t)(t0 + 1) * a.K};
+    float* const o[2] = {a.out + (size_t)t0 * a.n_rows, a.out + (size_t)(t0 + 1) * a.n_rows};
+    const float sc[2] = {1.0f, 1.0f};
+    matvec_rows<QUANT, KS, RPS, 2, NM>(a.w0, a.w1, a.K, a.n_rows, blockIdx.x * a.tile_rows, a.tile_rows, xr, o, sc);
+  } else {
+    const float* const xr[1] = {a.x + (size_t)t0 * a.K};
+    float* const o[1] = {a.out + (size_t)t0 * a.n_rows};
+    const float sc[1] = {1.0f};
+    matvec_rows<QUANT, KS, RPS, 1, NM>(a.w0, a.w1, a.K, a.n_rows, blockIdx.x * a.tile_rows, a.tile_rows, xr, o, sc);
+  }
+}
+
+}  // namespace xabe

@@ -1,0 +1,92 @@
+// Host-side state shared by the C-ABI translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/xabe_hip.h"
+
+namespace xabe {
+
+// Widths at which the regimes change hands.
+//   <= kFlatMaxTokens: flat per-pair kernels, no dispatch table
+//      (MOE_NARROW_DECODE_MAX, crates/xabe-cuda/src/kernels/moe.rs:213-229).
+//   >= kMfmaMinTokens: matrix-core grouped GEMM.  The reference switches its int8 path in at 8
+//      tokens (MMA_MIN_TOKENS); here the fp32 regime is kept through 63 so that every decode
+//      batch up to 32 sequences stays bit-identical to single-stream decode.
+constexpr size_t kFlatMaxTokens = 4;
+constexpr size_t kMfmaMinTokens = 64;
+constexpr size_t kRouteMaxExperts = 512;  // the routing wavefront holds 8 experts per lane
+
+int set_error(int status, const char* fmt, ...);
+int hip_error(hipError_t e, const char* what);
+std::string geometry_debug(const xabe_moe_geometry& g);
+
+#define XABE_HIP_TRY(expr)                                  \
+  do {                                                      \
+    hipError_t _e = (expr);                                 \
+    if (_e != hipSuccess) return ::xabe::hip_error(_e, #expr); \
+  } while (0)
+
+#define XABE_TRY(expr)            \
+  do {                            \
+    int _s = (expr);              \
+    if (_s != XABE_OK) return _s; \
+  } while (0)
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+}  // namespace xabe
+
+struct xabe_moe_kernels;
+struct xabe_moe_buffers;
+
+namespace xabe {
+// matrix-core regime (mfma.hip)
+bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int gate_q, int up_q, int down_q, bool routed);
+int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                                 xabe_quant_tensor up, xabe_quant_tensor down, const float* x);
+int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                       xabe_quant_tensor up, xabe_quant_tensor down, const float* x, float* out);
+
+}  // namespace xabe
+
+struct xabe_moe_kernels {
+  xabe_moe_geometry g;
+  bool tensor_cores;
+  bool exact_regime;
+  bool force_community;
+  int device;
+  int num_cus;
+};
+
+struct xabe_moe_buffers {
+  int scope;
+  bool mma;
+  xabe_moe_geometry g;
+  // lengths in elements
+  size_t n_topk, n_sorted, n_expert_blocks, n_inter, n_partial, n_shared_inter;
+  int32_t* topk_ids;
+  float* topk_weights;
+  int32_t* sorted_token_ids;
+  int32_t* expert_ids;
+  int32_t* bucket_live;
+  int32_t* expert_counts;
+  int32_t* num_tokens_post_pad;
+  int32_t* valid_tokens;
+  int32_t valid_published;
+  float* inter;         // [slot][intermediate] fp32 (decode regimes)
+  float* partial;       // [flat][hidden]
+  float* shared_inter;  // [token][intermediate]
+  // matrix-core regime staging
+  uint16_t* x_h;        // [token][hidden] fp16 activations
+  uint16_t* inter_h;    // [slot][intermediate] fp16
+  uint16_t* shared_inter_h;
+  int32_t* tile_list;   // device-built tile schedule
+  size_t n_tile_list;
+  size_t bytes;
+};

@@ -1,0 +1,425 @@
+// The small kernels around the expert contractions: RMSNorm, routing, dispatch
+// tables, combine, stand-alone dequantisation and the synthetic-stack generator.
+#pragma once
+
+#include "device_common.h"
+
+namespace xabe {
+
+// Sum over a 256-thread workgroup in a fixed order: the wavefront tree, then the four
+// wavefront totals ascending.  `scratch` holds 4 floats.
+__device__ __forceinline__ float block_sum_256(float v, float* scratch) {
+  v = group_sum<64>(v);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  const float total = ((scratch[0] + scratch[1]) + scratch[2]) + scratch[3];
+  __syncthreads();
+  return total;
+}
+
+// ---------------------------------------------------------------------------------
+// rms_norm_rows (crates/xabe-cuda/src/kernels/layer_ops.rs:129-151): every row of the
+// buffer, y = x * (1/sqrtf(mean(x^2) + eps)) * w.  grid = rows, 256 threads.
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__ x, const float* __restrict__ w,
+                                                        float* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[4];
+  const float* xr = x + (size_t)blockIdx.x * width;
+  float* o = out + (size_t)blockIdx.x * width;
+  float s = 0.0f;
+  for (int j = threadIdx.x; j < width; j += 256) {
+    const float v = xr[j];
+    s = __builtin_fmaf(v, v, s);
+  }
+  const float ss = block_sum_256(s, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  for (int j = threadIdx.x; j < width; j += 256) o[j] = xr[j] * inv * w[j];
+}
+
+// ---------------------------------------------------------------------------------
+// route (crates/xabe-cuda/src/kernels/moe.rs:1852-2036; CPU: crates/xabe-kernels/src/moe/router.rs:32-76).
+// One wavefront per token, four tokens per workgroup.  The arithmetic is the CPU
+// reference's, operation for operation, so the selected ids are the ones route_token
+// returns for these logits: max (order-free), e = exp(l - max), the sum of e taken
+// sequentially in index order, p = e / sum, top-k by (p descending, index ascending),
+// weights p / (sum of the selected p in selection order).
+// exp is evaluated in double and rounded once, which is the correctly rounded fp32 exp
+// except on a ~2^-29 fraction of inputs.
+// ---------------------------------------------------------------------------------
+constexpr int kRouteMaxPerLane = 8;  // 64 lanes x 8 = 512 experts
+
+__global__ void __launch_bounds__(256) k_route(const float* __restrict__ logits, const int* __restrict__ valid_tokens,
+                                                int num_experts, int top_k, int* __restrict__ topk_ids,
+                                                float* __restrict__ topk_weights) {
+  extern __shared__ float route_smem[];  // 4 x num_experts
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= *valid_tokens) return;
+  float* e_all = route_smem + (size_t)wave * num_experts;
+  const float* lg = logits + (size_t)t * num_experts;
+  const int per = (num_experts + 63) >> 6;
+
+  float l[kRouteMaxPerLane];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kRouteMaxPerLane; ++i) {
+    const int idx = i * 64 + lane;
+    l[i] = (i < per && idx < num_experts) ? lg[idx] : -INFINITY;
+    m = fmaxf(m, l[i]);
+  }
+  m = wave_max(m);
+#pragma unroll
+  for (int i = 0; i < kRouteMaxPerLane; ++i) {
+    const int idx = i * 64 + lane;
+    if (i < per && idx < num_experts) e_all[idx] = (float)exp((double)(l[i] - m));
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  // sequential sum, every lane redundantly (LDS broadcast reads)
+  float sum = -0.0f;
+  for (int i = 0; i < num_experts; ++i) sum += e_all[i];
+  float p[kRouteMaxPerLane];
+#pragma unroll
+  for (int i = 0; i < kRouteMaxPerLane; ++i) {
+    const int idx = i * 64 + lane;
+    p[i] = (i < per && idx < num_experts) ? e_all[idx] / sum : -1.0f;  // -1: never selected
+  }
+  // top-k: each round takes the (p max, idx min) over everything not yet taken
+  float sel_p = 0.0f;  // lane k keeps the k-th selected probability
+  int sel_i = 0;
+  for (int k = 0; k < top_k; ++k) {
+    float bp = -1.0f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < kRouteMaxPerLane; ++i) {
+      const int idx = i * 64 + lane;
+      if (p[i] > bp) { bp = p[i]; bi = idx; }  // ascending idx within a lane, strict > keeps the lower
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const float op = __shfl_xor(bp, off, 64);
+      const int oi = __shfl_xor(bi, off, 64);
+      if (op > bp || (op == bp && oi < bi)) { bp = op; bi = oi; }
+    }
+    if (lane == k) { sel_p = bp; sel_i = bi; }
+    if ((bi & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < kRouteMaxPerLane; ++i)
+        if (i == (bi >> 6)) p[i] = -1.0f;
+    }
+  }
+  // selected sum in selection order
+  float ssum = -0.0f;
+  for (int k = 0; k < top_k; ++k) ssum += __shfl(sel_p, k, 64);
+  if (lane < top_k) {
+    topk_ids[(size_t)t * top_k + lane] = sel_i;
+    topk_weights[(size_t)t * top_k + lane] = ssum > 0.0f ? sel_p / ssum : 1.0f / (float)top_k;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Dispatch tables (crates/xabe-cuda/src/kernels/moe.rs:2233-2366; CPU:
+// crates/xabe-kernels/src/moe/dispatch.rs:60-131).  Two launches of num_experts workgroups.
+//   count:   per-expert selection counts; whole-capacity sentinel / -1 / 0 fill.
+//   scatter: exclusive prefix of padded counts (recomputed per workgroup), then the
+//            expert's flat ids in ascending order, by a workgroup scan: no atomics,
+//            so the order is the CPU reference's.
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) k_align_count(const int* __restrict__ topk_ids, const int* __restrict__ valid_tokens,
+                                                      int top_k, int sorted_capacity, int expert_capacity,
+                                                      int* __restrict__ sorted_token_ids, int* __restrict__ expert_ids,
+                                                      int* __restrict__ bucket_live, int* __restrict__ expert_counts) {
+  __shared__ int red[4];
+  const int e = blockIdx.x;
+  const int numel = *valid_tokens * top_k;
+  int c = 0;
+  for (int i = threadIdx.x; i < numel; i += 256) c += topk_ids[i] == e;
+  for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) expert_counts[e] = red[0] + red[1] + red[2] + red[3];
+  // fill this workgroup's slice of the fixed-capacity tables
+  const int nb = gridDim.x;
+  for (int i = e * 256 + threadIdx.x; i < sorted_capacity; i += nb * 256) sorted_token_ids[i] = numel;
+  for (int i = e * 256 + threadIdx.x; i < expert_capacity; i += nb * 256) {
+    expert_ids[i] = -1;
+    bucket_live[i] = 0;
+  }
+}
+
+__global__ void __launch_bounds__(256) k_align_scatter(const int* __restrict__ topk_ids, const int* __restrict__ valid_tokens,
+                                                        const int* __restrict__ expert_counts, int top_k, int num_experts,
+                                                        int block_size, int sorted_capacity, int expert_capacity,
+                                                        int* __restrict__ sorted_token_ids, int* __restrict__ expert_ids,
+                                                        int* __restrict__ num_tokens_post_pad, int* __restrict__ bucket_live) {
+  __shared__ int s_wave[4];
+  __shared__ int s_base;
+  __shared__ int s_total;
+  const int e = blockIdx.x;
+  const int numel = *valid_tokens * top_k;
+  // exclusive prefix of padded counts below e, and the grand total
+  int below = 0, total = 0;
+  for (int i = threadIdx.x; i < num_experts; i += 256) {
+    const int padded = (expert_counts[i] + block_size - 1) / block_size * block_size;
+    total += padded;
+    if (i < e) below += padded;
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    below += __shfl_xor(below, off, 64);
+    total += __shfl_xor(total, off, 64);
+  }
+  if ((threadIdx.x & 63) == 0) s_wave[threadIdx.x >> 6] = below;
+  __syncthreads();
+  if (threadIdx.x == 0) s_base = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) s_wave[threadIdx.x >> 6] = total;
+  __syncthreads();
+  if (threadIdx.x == 0) s_total = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+  __syncthreads();
+  const int base = s_base;
+  if (e == 0 && threadIdx.x == 0) *num_tokens_post_pad = s_total;
+  const int count = expert_counts[e];
+  // this expert's blocks
+  const int nblk = (count + block_size - 1) / block_size;
+  for (int b = threadIdx.x; b < nblk; b += 256) {
+    const int blk = base / block_size + b;
+    if (blk < expert_capacity) {
+      expert_ids[blk] = e;
+      bucket_live[blk] = min(block_size, count - b * block_size);
+    }
+  }
+  // ordered placement: running offset + workgroup exclusive scan of the match flags
+  int running = 0;
+  for (int i0 = 0; i0 < numel; i0 += 256) {
+    const int i = i0 + threadIdx.x;
+    const int flag = (i < numel) && (topk_ids[i] == e);
+    const unsigned long long ballot = __ballot(flag);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
+    __syncthreads();
+    if (lane == 0) s_wave[wave] = __popcll(ballot);
+    __syncthreads();
+    int wave_base = 0;
+    for (int w = 0; w < wave; ++w) wave_base += s_wave[w];
+    const int chunk_total = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+    if (flag) {
+      const int slot = base + running + wave_base + before;
+      if (slot < sorted_capacity) sorted_token_ids[slot] = i;
+    }
+    running += chunk_total;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// moe_reduce (crates/xabe-cuda/src/kernels/moe.rs:4049-4065): out[t] = sum_k partial[t*K+k], ascending k.
+// grid (max_tokens, ceil(hidden/256)).
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) k_moe_reduce(const float* __restrict__ partial, const int* __restrict__ valid_tokens,
+                                                     int top_k, int hidden, float* __restrict__ out) {
+  const int t = blockIdx.x;
+  if (t >= *valid_tokens) return;
+  const int j = blockIdx.y * 256 + threadIdx.x;
+  if (j >= hidden) return;
+  const float* p = partial + (size_t)t * top_k * hidden + j;
+  float r = 0.0f;
+  for (int k = 0; k < top_k; ++k) r += p[(size_t)k * hidden];
+  out[(size_t)t * hidden + j] = r;
+}
+
+// ---------------------------------------------------------------------------------
+// moe_block_gate_and_combine (crates/xabe-engine/src/block/moe.rs:424-483):
+//   g = 1/(1+expf(-(w . normed[t])));  r = sum_k partial (ascending k);
+//   ffn_out = r + shexp*g;  l_out = ffn_out + residual.   grid (max_tokens, ceil(hidden/256)).
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) k_gate_and_combine(const float* __restrict__ w, const float* __restrict__ normed,
+                                                           const float* __restrict__ partial, const float* __restrict__ shexp,
+                                                           const float* __restrict__ residual, const int* __restrict__ valid_tokens,
+                                                           int top_k, int hidden, float* __restrict__ gate,
+                                                           float* __restrict__ routed, float* __restrict__ ffn_out,
+                                                           float* __restrict__ l_out) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  if (t >= *valid_tokens) return;
+  const size_t base = (size_t)t * hidden;
+  const float* xs = normed + base;
+  float s = 0.0f;
+  for (int j = threadIdx.x; j < hidden; j += 256) s = __builtin_fmaf(w[j], xs[j], s);
+  s = block_sum_256(s, scratch);
+  const float g = 1.0f / (1.0f + expf(-s));
+  if (threadIdx.x == 0 && blockIdx.y == 0) gate[t] = g;
+  const int j = blockIdx.y * 256 + threadIdx.x;
+  if (j >= hidden) return;
+  const float* p = partial + (size_t)t * top_k * hidden + j;
+  float r = 0.0f;
+  for (int k = 0; k < top_k; ++k) r += p[(size_t)k * hidden];
+  const float v = r + shexp[base + j] * g;
+  routed[base + j] = r;
+  ffn_out[base + j] = v;
+  l_out[base + j] = v + residual[base + j];
+}
+
+// dense_ffn_add_residual (crates/xabe-engine/src/block/dense_ffn.rs:1149-1175)
+__global__ void __launch_bounds__(256) k_add_residual(const float* __restrict__ ffn_out, const float* __restrict__ residual,
+                                                       const int* __restrict__ valid_tokens, int hidden,
+                                                       float* __restrict__ l_out) {
+  const int t = blockIdx.x;
+  if (t >= *valid_tokens) return;
+  const int j = blockIdx.y * 256 + threadIdx.x;
+  if (j >= hidden) return;
+  const size_t i = (size_t)t * hidden + j;
+  l_out[i] = ffn_out[i] + residual[i];
+}
+
+__global__ void __launch_bounds__(256) k_add_logit_bias(const float* __restrict__ bias, const int* __restrict__ valid_tokens,
+                                                         int num_experts, float* __restrict__ logits) {
+  const int t = blockIdx.x;
+  if (t >= *valid_tokens) return;
+  for (int e = threadIdx.x; e < num_experts; e += 256) logits[(size_t)t * num_experts + e] += bias[e];
+}
+
+// ---------------------------------------------------------------------------------
+// Stand-alone dequantisation, bit-identical to the CPU reference
+// (crates/xabe-kernels/src/quant.rs:62-69, :171-202): (d*sc)*q and q*d, each product rounded.
+// One thread per element.
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) k_dequant_q6k(const uint8_t* __restrict__ bytes, size_t n_elems, float* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_elems) return;
+  const uint8_t* b = bytes + (i >> 8) * kQ6KBytes;
+  const int n = (int)(i & 255);
+  const int half = n >> 7, lane = (n & 127) >> 5, l = n & 31;
+  const uint32_t qlb = b[half * 64 + (lane & 1) * 32 + l];
+  const uint32_t low4 = lane >= 2 ? qlb >> 4 : qlb & 0xF;
+  const uint32_t hi2 = (b[128 + half * 32 + l] >> (2 * lane)) & 3;
+  const int q = (int)(low4 | (hi2 << 4)) - 32;
+  const float sc = (float)(int8_t)b[192 + half * 8 + lane * 2 + (l >> 4)];
+  const float d = f16_bits_to_f32((uint32_t)b[208] | ((uint32_t)b[209] << 8));
+  const float dsc = d * sc;
+  out[i] = dsc * (float)q;
+}
+
+__global__ void __launch_bounds__(256) k_dequant_q8_0(const uint8_t* __restrict__ bytes, size_t n_elems, float* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_elems) return;
+  const uint8_t* b = bytes + (i >> 5) * kQ8Bytes;
+  const float d = f16_bits_to_f32((uint32_t)b[0] | ((uint32_t)b[1] << 8));
+  out[i] = (float)(int8_t)b[2 + (i & 31)] * d;
+}
+
+// ---------------------------------------------------------------------------------
+// Synthetic stacks: one thread per 256-element chunk.  Integer Irwin-Hall(12) normal
+// approximation over a per-chunk xorshift64* stream, then the reference's amax
+// quantizers (crates/xabe-kernels/src/quant.rs:75-88, :495-567).
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+__device__ __forceinline__ uint64_t xorshift_next(uint64_t& s) {
+  uint64_t x = s;
+  x ^= x >> 12;
+  x ^= x << 25;
+  x ^= x >> 27;
+  s = x;
+  return x * 0x2545F4914F6CDD1Dull;
+}
+__device__ __forceinline__ uint64_t chunk_state(uint64_t seed, size_t chunk) {
+  const uint64_t st = splitmix64(seed + (uint64_t)chunk * 0x9E3779B97F4A7C15ull);
+  return st == 0 ? 0x9E3779B97F4A7C15ull : st;
+}
+__device__ __forceinline__ float synth_value(uint64_t& st, float sigma) {
+  uint32_t s = 0;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    const uint64_t v = xorshift_next(st);
+    s += (uint32_t)(v & 0xffff) + (uint32_t)((v >> 16) & 0xffff) + (uint32_t)((v >> 32) & 0xffff) + (uint32_t)(v >> 48);
+  }
+  const float z = (float)(2 * (int32_t)s - 12 * 65535) * (1.0f / 131072.0f);
+  return sigma * z;
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float v) {
+  return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+__device__ __forceinline__ float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+__global__ void __launch_bounds__(64) k_synth_f32(uint64_t seed, size_t n, float sigma, float* __restrict__ out) {
+  const size_t c = (size_t)blockIdx.x * 64 + threadIdx.x;
+  if (c * 256 >= n) return;
+  uint64_t st = chunk_state(seed, c);
+  const size_t m = min((size_t)256, n - c * 256);
+  for (size_t i = 0; i < m; ++i) out[c * 256 + i] = synth_value(st, sigma);
+}
+
+__global__ void __launch_bounds__(64) k_synth_q6k(uint64_t seed, size_t chunks, float sigma, uint8_t* __restrict__ out) {
+  const size_t c = (size_t)blockIdx.x * 64 + threadIdx.x;
+  if (c >= chunks) return;
+  // pass 1: group and global amax
+  uint64_t st = chunk_state(seed, c);
+  float gamax[16];
+  float amax = 0.0f;
+#pragma unroll
+  for (int g = 0; g < 16; ++g) {
+    float a = 0.0f;
+    for (int k = 0; k < 16; ++k) a = fmaxf(a, fabsf(synth_value(st, sigma)));
+    gamax[g] = a;
+    amax = fmaxf(amax, a);
+  }
+  const float d = amax > 0.0f ? amax / (32.0f * 127.0f) : 0.0f;
+  uint8_t* blk = out + c * kQ6KBytes;
+  for (int i = 0; i < 192; ++i) blk[i] = 0;
+  // pass 2: regenerate, quantize, pack (group g covers positions 16g..16g+15)
+  st = chunk_state(seed, c);
+#pragma unroll
+  for (int g = 0; g < 16; ++g) {
+    int sc = 0;
+    if (d > 0.0f) sc = (int)clampf(roundf(gamax[g] / (d * 32.0f)), 0.0f, 127.0f);
+    blk[192 + g] = (uint8_t)(int8_t)sc;
+    const float denom = d * (float)sc;
+    const int half = g >> 3, lane = (g >> 1) & 3, is = g & 1;
+    for (int k = 0; k < 16; ++k) {
+      const float v = synth_value(st, sigma);
+      const int l = is * 16 + k;
+      int code = 0;
+      if (denom != 0.0f) code = (int)clampf(roundf(v / denom), -32.0f, 31.0f);
+      const uint32_t raw = (uint32_t)(code + 32);
+      blk[128 + half * 32 + l] |= (uint8_t)((raw >> 4) << (lane * 2));
+      const int qi = half * 64 + (lane & 1) * 32 + l;
+      blk[qi] |= (uint8_t)(lane >= 2 ? (raw & 0xF) << 4 : (raw & 0xF));
+    }
+  }
+  const uint16_t dh = f32_to_f16_bits(d);
+  blk[208] = (uint8_t)(dh & 0xff);
+  blk[209] = (uint8_t)(dh >> 8);
+}
+
+__global__ void __launch_bounds__(64) k_synth_q8_0(uint64_t seed, size_t chunks, float sigma, uint8_t* __restrict__ out) {
+  const size_t c = (size_t)blockIdx.x * 64 + threadIdx.x;
+  if (c >= chunks) return;
+  uint64_t st = chunk_state(seed, c);
+  for (int b = 0; b < 8; ++b) {
+    float v[32];
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      v[j] = synth_value(st, sigma);
+      amax = fmaxf(amax, fabsf(v[j]));
+    }
+    const float d = amax / 127.0f;
+    const float inv_d = d != 0.0f ? 1.0f / d : 0.0f;
+    uint8_t* blk = out + (c * 8 + b) * kQ8Bytes;
+    const uint16_t dh = f32_to_f16_bits(d);
+    blk[0] = (uint8_t)(dh & 0xff);
+    blk[1] = (uint8_t)(dh >> 8);
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      float q = roundf(v[j] * inv_d);
+      q = clampf(q, -128.0f, 127.0f);
+      blk[2 + j] = (uint8_t)(int8_t)(int)q;
+    }
+  }
+}
+
+}  // namespace xabe
