@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized MoE block on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the MoE block over one batch: 3 tokens (three concurrent sequences, one token
+each), 256 experts top-8 + 1 shared, hidden 2048, expert width 512, Q6_K experts, Q8_0 router and
+shared expert -- BASELINE.json configs[1].  Successive steps run on different, independently seeded
+layers (--layers, default 16, 10.7 GB) so that a step's weights come from HBM and not from the
+256 MB Infinity Cache.  Inputs are resident in HBM before the timed region starts.
+
+Prints one JSON line: whole-job tokens/s, the roofline of the dominant kernel (routed gate/up GEMV,
+algorithmic bytes / measured launch duration against the 8 TB/s HBM peak) and the CPU oracle timed
+on this host's cores."""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+EXPERT_MATRIX_BYTES = 512 * 2048 // 256 * 210   # one Q6_K [512 x 2048] matrix: 860160 B
+SHARED_BYTES = 3 * (512 * 2048 // 32 * 34)      # shared expert, Q8_0
+ROUTER_BYTES = 256 * 2048 // 32 * 34            # router, Q8_0
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=320)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--layers", type=int, default=16, help="independent weight sets rotated through")
+    ap.add_argument("--tokens", type=int, default=3)
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a hipGraph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    import llmxabe_amd as X
+
+    torch.cuda.set_device(0)
+    T = args.tokens
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
+    L = args.layers
+
+    layers = []
+    for l in range(L):
+        layers.append(make_layer_device_only(X, g, seed=10_000 + 100 * l))
+    x = X.synth_normal_f32(99, T * 2048, 1.0).view(T, 2048)   # fp32 N(0,1) activations, resident in HBM
+    blk = X.MoeBlock(g)
+    blk.publish_tokens(T)
+    ffn_out = torch.zeros_like(x)
+    l_out = torch.zeros_like(x)
+
+    def one_pass(i):
+        blk.forward(layers[i % L], x, T, ffn_out, l_out)
+
+    # ---- timed region: K steps, W warmup ----
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(L):
+            one_pass(i)
+        stream.synchronize()
+        graph = None
+        if not args.no_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(L):
+                    one_pass(i)
+        reps_w = max(1, (args.warmup + L - 1) // L)
+        reps = max(1, (args.steps + L - 1) // L)
+        steps = reps * L
+        for _ in range(reps_w):
+            graph.replay() if graph else [one_pass(i) for i in range(L)]
+        stream.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            graph.replay() if graph else [one_pass(i) for i in range(L)]
+        stream.synchronize()
+        dt = time.perf_counter() - t0
+    ms_per_step = dt / steps * 1e3
+    tokens_per_s = T * steps / dt
+
+    # ---- algorithmic bytes of one step (distinct experts from topk_ids of each layer) ----
+    distinct = []
+    with torch.cuda.stream(stream):
+        for i in range(L):
+            one_pass(i)
+            stream.synchronize()
+            ids = blk.buffers().topk_ids().cpu().numpy().reshape(T, 8)
+            distinct.append(len(np.unique(ids)))
+    d_active = float(np.mean(distinct))
+    step_bytes = d_active * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES + 16384 + T * 2048 * 4 * 3
+    step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- dominant kernel: routed gate/up GEMV (two of three expert matrices) ----
+    k = X.MoeKernels(g)
+    b = k.buffers()
+    k.set_valid_tokens(b, T)
+    normed = torch.empty_like(x)
+    logits = torch.empty(T, 256, device="cuda")
+    per_layer_bytes = []
+    with torch.cuda.stream(stream):
+        def stage0(i):
+            w = layers[i % L]
+            k.grouped_forward_stage(b, w.gate_exps, w.up_exps, w.down_exps, normed, 0)
+
+        # one routing decision per layer, fixed for the measurement
+        w0 = layers[0]
+        X.LayerOpsKernels.rms_norm(x, w0.post_norm, normed, T, 2048, 1e-6)
+        k.router_logits(b, w0.router, w0.router_quant, normed, logits)
+        k.route_and_dispatch(b, logits)
+        stream.synchronize()
+        pairs = T * 8
+        kern_bytes = pairs * 2 * EXPERT_MATRIX_BYTES  # the flat kernel streams gate+up once per (token, k) pair
+        kgraph = torch.cuda.CUDAGraph()
+        for i in range(L):
+            stage0(i)
+        stream.synchronize()
+        with torch.cuda.graph(kgraph, stream=stream):
+            for i in range(L):
+                stage0(i)
+        kgraph.replay()
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        kreps = 20
+        e0.record(stream)
+        for _ in range(kreps):
+            kgraph.replay()
+        e1.record(stream)
+        e1.synchronize()
+        kern_us = e0.elapsed_time(e1) * 1e3 / (kreps * L)
+    achieved = kern_bytes / (kern_us * 1e-6) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("k_expert_flat_gateup_b3_bytes_per_launch")
+        except Exception:
+            traffic = None
+
+    out = {
+        "metric": "MoE-block tokens/s at 1 GPU; decode HBM GB/s %peak; prefill MFMA util %",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": reps_w * L,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "moe_block_decode_b3" if T == 3 else f"moe_block_decode_b{T}", "tokens": T,
+                   "num_experts": 256, "top_k": 8, "hidden": 2048, "intermediate": 512, "expert_quant": "Q6_K",
+                   "shared_and_router_quant": "Q8_0", "layers_rotated": L, "launch": "eager" if args.no_graph else "hipGraph"},
+        "decode": {"distinct_experts_per_step": d_active, "algorithmic_bytes_per_step": step_bytes,
+                   "block_gbps": step_gbps, "block_frac_of_hbm_peak": step_gbps / HBM_PEAK_GBPS,
+                   "roofline_tokens_per_s": T / (step_bytes / (HBM_PEAK_GBPS * 1e9)),
+                   "frac_of_roofline": tokens_per_s / (T / (step_bytes / (HBM_PEAK_GBPS * 1e9)))},
+        "roofline": {"kernel": "k_expert_flat<Q6_K,K=2048,gate+up>", "bound": "hbm", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
+                     "algorithmic_bytes_per_launch": kern_bytes, "launch_us": kern_us},
+    }
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(layers[0], g, x, T, args.cpu_seconds)
+    print(json.dumps(out))
+    return 0
+
+
+def make_layer_device_only(X, g, seed):
+    """Seeded device tensors of one layer (same definition as tests/util.make_layer, no host copy)."""
+    ROLE = dict(post_norm=1, router=2, gate=3, up=4, down=5, shared_gate_inp=6, sgate=7, sup=8, sdown=9)
+    E, H, I = g.num_experts, g.hidden, g.intermediate
+    n = E * I * H
+    q6, q8 = X.ExpertQuant.Q6K, X.ExpertQuant.Q8_0
+    qt = lambda q, role, count: X.QuantTensor(X.synth_quant(q, seed + ROLE[role], count, 0.02), q)
+    return X.MoeLayerWeights(
+        1.0 + X.synth_normal_f32(seed + ROLE["post_norm"], H, 0.1),
+        X.synth_quant(q8, seed + ROLE["router"], E * H, 0.02), q8,
+        qt(q6, "gate", n), qt(q6, "up", n), qt(q6, "down", n),
+        X.synth_normal_f32(seed + ROLE["shared_gate_inp"], H, 0.02),
+        qt(q8, "sgate", I * H), qt(q8, "sup", I * H), qt(q8, "sdown", I * H))
+
+
+def cpu_baseline(w, g, x, T, budget_s):
+    """The CPU oracle (a C port of the reference's scalar path) on this host: the same block, same
+    layer-0 weights, same T tokens, repeated until about `budget_s` seconds of CPU work are spent."""
+    import oracle
+
+    c = lambda t: t.cpu().numpy()
+    host = oracle.MoeWeights(
+        num_experts=g.num_experts, top_k=g.experts_per_token, hidden=g.hidden, intermediate=g.intermediate, eps=1e-6,
+        post_norm=c(w.post_norm), router_f32=None, router_q8=c(w.router), gate_exps=c(w.gate_exps.bytes),
+        up_exps=c(w.up_exps.bytes), down_exps=c(w.down_exps.bytes), shared_gate_inp=c(w.shared_gate_inp),
+        shared_gate=c(w.shared_gate.bytes), shared_up=c(w.shared_up.bytes), shared_down=c(w.shared_down.bytes))
+    xs = c(x)[:T]
+
+    def run(threads, budget):
+        n, t0, deq, mv = 0, time.perf_counter(), 0.0, 0.0
+        while True:
+            r = oracle.moe_block_forward(host, xs, threads=threads)
+            n += 1
+            deq += r.seconds_dequant
+            mv += r.seconds_matvec
+            el = time.perf_counter() - t0
+            if el >= budget or n >= 200:
+                return n, el, deq, mv
+
+    n1, el1, deq1, mv1 = run(1, budget_s * 0.7)
+    cores = min(oracle.num_threads(), 16)
+    nt, elt, _, _ = run(cores, budget_s * 0.3)
+    return {"value": T * n1 / el1, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"{n1} passes of the same {T}-token block on layer 0 (dequantise selected experts + sequential "
+                      f"fp32 matvecs), {el1:.1f} s; dequant {deq1 / n1 * 1e3:.0f} ms + matvec {mv1 / n1 * 1e3:.0f} ms per pass",
+            "openmp": {"value": T * nt / elt, "cores": cores, "passes": nt, "seconds": elt}}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

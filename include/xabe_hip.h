@@ -150,6 +150,12 @@ int xabe_moe_route_and_dispatch(const xabe_moe_kernels* k, void* stream, xabe_mo
 int xabe_moe_grouped_forward_partial(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b,
                                      xabe_quant_tensor gate, xabe_quant_tensor up, xabe_quant_tensor down,
                                      const float* hidden_states, size_t hidden_states_len);
+/* One half of grouped_forward_partial on its own: stage 0 = gate/up + SwiGLU (fills the intermediate),
+ * stage 1 = down (fills `partial`).  For measurement: the reference's bench times the stages of the
+ * path separately (crates/xabe-cuda/src/bin/bench_moe.rs:140-334). */
+int xabe_moe_grouped_forward_stage(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                                   xabe_quant_tensor up, xabe_quant_tensor down, const float* hidden_states,
+                                   size_t hidden_states_len, int stage);
 /* MoeKernels::grouped_forward_partial_with_shared (M:6190-6335).  `*fused` = 1 when the shared
  * expert rode the routed launches, 0 (nothing launched) when the pass is not covered. */
 int xabe_moe_grouped_forward_partial_with_shared(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b,

@@ -76,6 +76,7 @@ _SIGNATURES = {
     "xabe_moe_build_dispatch": (C.c_int, [vp, vp, vp]),
     "xabe_moe_route_and_dispatch": (C.c_int, [vp, vp, vp, vp, sz]),
     "xabe_moe_grouped_forward_partial": (C.c_int, [vp, vp, vp, QuantTensorC, QuantTensorC, QuantTensorC, vp, sz]),
+    "xabe_moe_grouped_forward_stage": (C.c_int, [vp, vp, vp, QuantTensorC, QuantTensorC, QuantTensorC, vp, sz, C.c_int]),
     "xabe_moe_grouped_forward_partial_with_shared": (C.c_int, [vp, vp, vp] + [QuantTensorC] * 6 + [vp, sz, vp, sz, C.POINTER(C.c_int)]),
     "xabe_moe_grouped_forward": (C.c_int, [vp, vp, vp, QuantTensorC, QuantTensorC, QuantTensorC, vp, sz, vp, sz]),
     "xabe_moe_shared_expert": (C.c_int, [vp, vp, vp, QuantTensorC, QuantTensorC, QuantTensorC, vp, sz, vp, sz]),

@@ -482,8 +482,9 @@ static int check_routed_stacks(const xabe_moe_kernels* k, xabe_quant_tensor gate
   return XABE_OK;
 }
 
+// stages: bit 0 = gate/up + SwiGLU, bit 1 = down
 static int routed_fp32(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
-                       xabe_quant_tensor up, xabe_quant_tensor down, const float* x) {
+                       xabe_quant_tensor up, xabe_quant_tensor down, const float* x, int stages = 3) {
   const xabe_moe_geometry& g = k->g;
   const bool flat = flat_regime(k);
   const size_t units = flat ? xabe_moe_geometry_max_flat_pairs(&g) : b->n_expert_blocks;
@@ -497,7 +498,8 @@ static int routed_fp32(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffer
   a.out = b->inter;
   a.K = (int)g.hidden;
   a.n_rows = (int)g.intermediate;
-  XABE_TRY(launch_expert(k, flat ? kFlat : kBlock, gate.quant, 2, a, units, flat ? units : live, s));
+  if (stages & 1) XABE_TRY(launch_expert(k, flat ? kFlat : kBlock, gate.quant, 2, a, units, flat ? units : live, s));
+  if (!(stages & 2)) return XABE_OK;
   a.w0 = static_cast<const uint8_t*>(down.bytes);
   a.w1 = nullptr;
   a.expert_bytes = expert_elems / xabe_expert_quant_block_elements(down.quant) * xabe_expert_quant_block_bytes(down.quant);
@@ -519,6 +521,19 @@ int xabe_moe_grouped_forward_partial(const xabe_moe_kernels* k, void* stream, xa
   if (!flat_regime(k) && mfma_supported(k, b, gate.quant, up.quant, down.quant, true))
     return mfma_grouped_forward_partial(k, as_stream(stream), b, gate, up, down, hidden_states);
   return routed_fp32(k, as_stream(stream), b, gate, up, down, hidden_states);
+}
+
+int xabe_moe_grouped_forward_stage(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                                   xabe_quant_tensor up, xabe_quant_tensor down, const float* hidden_states,
+                                   size_t hidden_states_len, int stage) {
+  if (!k || !b || !hidden_states) return set_error(XABE_ERR_INVALID_ARGUMENT, "grouped_forward_stage: null pointer");
+  if (stage != 0 && stage != 1) return set_error(XABE_ERR_INVALID_ARGUMENT, "grouped_forward_stage: stage must be 0 or 1");
+  XABE_TRY(require_routed(b, "grouped_forward_stage"));
+  XABE_TRY(check_routed_stacks(k, gate, up, down));
+  XABE_TRY(check_len("hidden_states", k->g.max_tokens * k->g.hidden, hidden_states_len));
+  if (!flat_regime(k) && mfma_supported(k, b, gate.quant, up.quant, down.quant, true))
+    return set_error(XABE_ERR_MMA, "grouped_forward_stage: the matrix-core regime has no separable stages");
+  return routed_fp32(k, as_stream(stream), b, gate, up, down, hidden_states, stage == 0 ? 1 : 2);
 }
 
 static int check_shared_stacks(const xabe_moe_kernels* k, xabe_quant_tensor gate, xabe_quant_tensor up,

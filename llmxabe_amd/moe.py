@@ -235,6 +235,10 @@ class MoeKernels:
         check(_ffi.lib().xabe_moe_grouped_forward_partial(self._h, _stream(), buffers._h, gate._c(), up._c(), down._c(),
                                                           _ptr(hidden_states), hidden_states.numel()))
 
+    def grouped_forward_stage(self, buffers, gate, up, down, hidden_states, stage: int):
+        check(_ffi.lib().xabe_moe_grouped_forward_stage(self._h, _stream(), buffers._h, gate._c(), up._c(), down._c(),
+                                                        _ptr(hidden_states), hidden_states.numel(), stage))
+
     def grouped_forward_partial_with_shared(self, buffers, gate, up, down, shared_gate, shared_up, shared_down,
                                             hidden_states, out) -> bool:
         fused = C.c_int(0)
