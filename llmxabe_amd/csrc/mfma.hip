@@ -1,21 +1,427 @@
-// Matrix-core (MFMA) regime for prefill widths.
+// Matrix-core regime for prefill widths: a grouped GEMM over expert-sorted tokens that
+// dequantises Q6_K / Q8_0 weight tiles into LDS as fp16 and feeds v_mfma_f32_32x32x16_f16.
+// Takes the place of the reference's int8 tensor-core family
+// (crates/xabe-cuda/src/kernels/moe.rs:1316-1819, :2901-2943, :3152-3373) and of its
+// int8 shared-expert path (moe.rs:6389-6476); one prologue per format feeds the same
+// MFMA body for gate, up and down, so there is no per-format asymmetry.
+//
+// Work decomposition.  A workgroup (4 wavefronts, 2x2) owns a 128-token x 128-weight-row
+// tile and walks the contraction in steps of 128.  For gate/up the 128 weight rows are 64
+// gate rows and the matching 64 up rows, so SwiGLU happens in registers.  Token tiles come
+// from a device-built list with one entry per 128-slot chunk of every *active* expert's
+// run of the dispatch table: experts with no tokens cost nothing, whatever the skew.
+// Workgroups are persistent and stride over (token tile, row tile) items.
+//
+// Numerics.  Operands are fp16: activations rounded once; weights are (code - offset) exactly,
+// times fp16(d * sc * 256) -- the 2^8 keeps small scales out of the fp16 subnormal range and
+// is divided out in the epilogue.  Accumulation is fp32 in the MFMA.  Each output element
+// depends only on its own token row and weight row in a fixed contraction order, so a token's
+// row is the same bits wherever it sits in a batch of this regime.
+#include <string.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "device_common.h"
 #include "host_common.h"
 
 namespace xabe {
 
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int kBM = 128;          // token rows per tile
+constexpr int kBR = 128;          // weight rows per tile
+constexpr int kBK = 128;          // contraction elements per step
+constexpr int kLd = kBK + 8;      // LDS row stride in halfs (272 B: 16-B reads are conflict-free)
+constexpr float kWScale = 256.0f;
+constexpr float kWScaleInv = 1.0f / 256.0f;
+
+struct MfmaArgs {
+  const uint8_t* w0;            // gate (NM=2) or down (NM=1) stack
+  const uint8_t* w1;            // up stack (NM=2)
+  size_t expert_bytes;          // bytes of one expert in a stack
+  const _Float16* a;            // activations, row-major [*][K]
+  void* out;                    // NM=2: fp16 [*][n_rows]; NM=1: fp32 [*][n_rows]
+  const int* valid_tokens;
+  const int* sorted_token_ids;
+  const float* topk_weights;
+  const int* tile_list;         // [0] = tile count; entry i at 4+4i: expert, first slot, live rows
+  int K;                        // contraction length
+  int n_rows;                   // output columns per token (rows of one weight matrix)
+  int top_k;
+};
+
+// ---- prologues: one 32-element unit of one weight row -> 32 halfs in LDS -----------------
+__device__ __forceinline__ uint4 pack8(uint32_t c0, uint32_t c1, half2v off, half2v s) {
+  // c0, c1: eight byte codes; returns eight halfs (code + 1024 - off) * s
+  uint32_t p[4];
+  p[0] = __builtin_amdgcn_perm(0x64646464u, c0, 0x04010400u);
+  p[1] = __builtin_amdgcn_perm(0x64646464u, c0, 0x04030402u);
+  p[2] = __builtin_amdgcn_perm(0x64646464u, c1, 0x04010400u);
+  p[3] = __builtin_amdgcn_perm(0x64646464u, c1, 0x04030402u);
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    half2v v = __builtin_bit_cast(half2v, p[i]);
+    v = (v + off) * s;
+    o[i] = __builtin_bit_cast(uint32_t, v);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// Q6_K unit (half h of a superblock, l8): codes at j*32 + l8*8 + i of that half.
+__device__ __forceinline__ void q6_unit_to_lds(const Q6Raw& r, int l8, _Float16* brow) {
+  const int is8 = (l8 >> 1) * 8;
+  const uint32_t slo = r.sc0 >> is8, shi = r.sc1 >> is8;
+  const float d = f16_bits_to_f32(r.dh) * kWScale;
+  const float ds[4] = {d * (float)(int8_t)(slo & 0xff), d * (float)(int8_t)((slo >> 16) & 0xff),
+                       d * (float)(int8_t)(shi & 0xff), d * (float)(int8_t)((shi >> 16) & 0xff)};
+  uint32_t c[2][4];
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    const uint32_t a = w ? r.qa1 : r.qa0, b = w ? r.qb1 : r.qb0, h = w ? r.qh1 : r.qh0;
+    c[w][0] = (a & 0x0F0F0F0Fu) | ((h << 4) & 0x30303030u);
+    c[w][1] = (b & 0x0F0F0F0Fu) | ((h << 2) & 0x30303030u);
+    c[w][2] = ((a >> 4) & 0x0F0F0F0Fu) | (h & 0x30303030u);
+    c[w][3] = ((b >> 4) & 0x0F0F0F0Fu) | ((h >> 2) & 0x30303030u);
+  }
+  const half2v off = {(_Float16)-1056.0f, (_Float16)-1056.0f};  // 1024 (perm bias) + 32 (code centre)
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const _Float16 sh = (_Float16)ds[j];
+    const half2v s = {sh, sh};
+    *reinterpret_cast<uint4*>(brow + j * 32 + l8 * 8) = pack8(c[0][j], c[1][j], off, s);
+  }
+}
+
+// Q8_0 unit: one 34-byte block -> 32 consecutive halfs.
+__device__ __forceinline__ void q8_unit_to_lds(const Q8Raw& r, _Float16* bdst) {
+  const _Float16 sh = (_Float16)(f16_bits_to_f32(r.dh) * kWScale);  // exact: d is fp16, scaled by 2^8
+  const half2v s = {sh, sh};
+  const half2v off = {(_Float16)-1152.0f, (_Float16)-1152.0f};      // 1024 (perm bias) + 128 (sign flip)
+#pragma unroll
+  for (int w = 0; w < 4; ++w)
+    reinterpret_cast<uint4*>(bdst)[w] = pack8(r.q[2 * w] ^ 0x80808080u, r.q[2 * w + 1] ^ 0x80808080u, off, s);
+}
+
+template <int QUANT>
+struct WRaw {
+  typename std::conditional<QUANT == kQ6K, Q6Raw, Q8Raw>::type u[2];
+};
+
+template <int QUANT, int NM, bool ROUTED>
+__global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
+  // 71 KB of LDS per workgroup (two per CU): dynamic, since the static limit is 64 KB
+  extern __shared__ __attribute__((aligned(16))) uint8_t mfma_smem[];
+  _Float16* sA = reinterpret_cast<_Float16*>(mfma_smem);
+  _Float16* sB = sA + kBM * kLd;
+  int* sArow = reinterpret_cast<int*>(sB + kBR * kLd);  // activation row index of each tile row
+  int* sOrow = sArow + kBM;                             // output row index, or -1 for a dead row
+  float* sScale = reinterpret_cast<float*>(sOrow + kBM);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int valid = *a.valid_tokens;
+  const int n_ntiles = a.n_rows / (NM == 2 ? 64 : 128);
+  const int n_mtiles = ROUTED ? a.tile_list[0] : (valid + kBM - 1) / kBM;
+  const int total = n_mtiles * n_ntiles;
+  const int nks = a.K / kBK;
+  const size_t row_bytes = QUANT == kQ6K ? (size_t)(a.K / 256) * kQ6KBytes : (size_t)(a.K / 32) * kQ8Bytes;
+
+  // dequant mapping: unit u of LDS weight rows rb0 and rb0 + 64
+  const int du = tid & 3, rb0 = tid >> 2;
+
+  for (int item = blockIdx.x; item < total; item += gridDim.x) {
+    const int mt = item / n_ntiles, nt = item % n_ntiles;
+    int e = 0, m0 = mt * kBM, rows = min(kBM, valid - mt * kBM);
+    if (ROUTED) {
+      e = a.tile_list[4 + 4 * mt];
+      m0 = a.tile_list[4 + 4 * mt + 1];
+      rows = a.tile_list[4 + 4 * mt + 2];
+    }
+    __syncthreads();  // the previous item is done with the row tables
+    if (tid < kBM) {
+      int arow = 0, orow = -1;
+      float sc = 1.0f;
+      if (tid < rows) {
+        if (ROUTED) {
+          const int slot = m0 + tid;
+          const int flat = a.sorted_token_ids[slot];
+          if (NM == 2) { arow = flat / a.top_k; orow = slot; }
+          else { arow = slot; orow = flat; sc = a.topk_weights[flat]; }
+        } else {
+          arow = orow = m0 + tid;
+        }
+      }
+      sArow[tid] = arow;
+      sOrow[tid] = orow;
+      sScale[tid] = sc;
+    }
+    __syncthreads();
+
+    // weight rows this thread dequantises
+    const uint8_t* wrow[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int rb = rb0 + 64 * i;
+      const uint8_t* base;
+      int wr;
+      if (NM == 2) {
+        const int half_n = rb >> 6, which = (rb >> 5) & 1, c = rb & 31;
+        base = which ? a.w1 : a.w0;
+        wr = nt * 64 + half_n * 32 + c;
+      } else {
+        base = a.w0;
+        wr = nt * 128 + rb;
+      }
+      wrow[i] = base + (size_t)e * a.expert_bytes + (size_t)wr * row_bytes;
+    }
+    // activation chunks this thread stages: 8 x 16 bytes per step
+    const _Float16* arow_ptr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int c = tid + 256 * i;
+      arow_ptr[i] = a.a + (size_t)sArow[c >> 4] * a.K + (c & 15) * 8;
+    }
+
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    uint4 areg[8];
+    WRaw<QUANT> wreg;
+    auto load_step = [&](int ks) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const uint4*>(arow_ptr[i] + (size_t)ks * kBK);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if constexpr (QUANT == kQ6K) {
+          // step ks covers half (ks & 1) of superblock ks >> 1
+          const uint8_t* p = wrow[i] + (size_t)(ks >> 1) * kQ6KBytes;
+          const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
+          q6_load(p - mis, mis, ks & 1, du, wreg.u[i]);
+        } else {
+          const uint8_t* p = wrow[i] + (size_t)(ks * 4 + du) * kQ8Bytes;
+          const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
+          q8_load(p - mis, mis, wreg.u[i]);
+        }
+      }
+    };
+    load_step(0);
+    for (int ks = 0; ks < nks; ++ks) {
+      __syncthreads();  // everyone has finished reading the previous step's tiles
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int c = tid + 256 * i;
+        *reinterpret_cast<uint4*>(&sA[(c >> 4) * kLd + (c & 15) * 8]) = areg[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int rb = rb0 + 64 * i;
+        if constexpr (QUANT == kQ6K) q6_unit_to_lds(wreg.u[i], du, &sB[rb * kLd]);
+        else q8_unit_to_lds(wreg.u[i], &sB[rb * kLd + du * 32]);
+      }
+      __syncthreads();
+      if (ks + 1 < nks) load_step(ks + 1);  // in flight while the matrix cores work
+      const _Float16* pa = &sA[(wm * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
+      const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
+#pragma unroll
+      for (int kk = 0; kk < kBK / 16; ++kk) {
+        const half8 a0 = *reinterpret_cast<const half8*>(pa + kk * 16);
+        const half8 a1 = *reinterpret_cast<const half8*>(pa + 32 * kLd + kk * 16);
+        const half8 b0 = *reinterpret_cast<const half8*>(pb + kk * 16);
+        const half8 b1 = *reinterpret_cast<const half8*>(pb + 32 * kLd + kk * 16);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b0, acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b1, acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc[1][1], 0, 0, 0);
+      }
+    }
+
+    // epilogue.  acc[mi][ni][v]: tile row (v/4)*8 + (lane/32)*4 + v%4, tile column lane%32
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int r = wm * 64 + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+        const int orow = sOrow[r];
+        if (orow < 0) continue;
+        if (NM == 2) {
+          const int col = nt * 64 + wn * 32 + (lane & 31);
+          const float g = acc[mi][0][v] * kWScaleInv, u = acc[mi][1][v] * kWScaleInv;
+          static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_f(g) * u);
+        } else {
+          const float sc = sScale[r];
+#pragma unroll
+          for (int ni = 0; ni < 2; ++ni) {
+            const int col = nt * 128 + wn * 64 + ni * 32 + (lane & 31);
+            static_cast<float*>(a.out)[(size_t)orow * a.n_rows + col] = sc * (acc[mi][ni][v] * kWScaleInv);
+          }
+        }
+      }
+    }
+  }
+}
+
+// fp32 -> fp16 activations for live rows; rows past `valid` are left alone.
+__global__ void __launch_bounds__(256) k_to_f16_rows(const float* __restrict__ x, const int* __restrict__ valid_tokens,
+                                                      int width, _Float16* __restrict__ out) {
+  const int t = blockIdx.x;
+  if (t >= *valid_tokens) return;
+  const float4* src = reinterpret_cast<const float4*>(x + (size_t)t * width);
+  uint2* dst = reinterpret_cast<uint2*>(out + (size_t)t * width);
+  for (int j = threadIdx.x; j < width / 4; j += 256) {
+    const float4 v = src[j];
+    const half2v lo = {(_Float16)v.x, (_Float16)v.y}, hi = {(_Float16)v.z, (_Float16)v.w};
+    dst[j] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+  }
+}
+
+// Token-tile list: one entry per 128-slot chunk of each active expert's run.  One workgroup.
+__global__ void __launch_bounds__(256) k_build_tiles(const int* __restrict__ expert_counts, int num_experts, int block_size,
+                                                      int capacity, int* __restrict__ tile_list) {
+  __shared__ int s_base[513], s_tiles[513];
+  // exclusive prefixes, serially by one thread per array (num_experts <= 512)
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int e = 0; e < num_experts; ++e) {
+      s_base[e] = acc;
+      acc += (expert_counts[e] + block_size - 1) / block_size * block_size;
+    }
+  }
+  if (threadIdx.x == 64) {
+    int acc = 0;
+    for (int e = 0; e < num_experts; ++e) {
+      s_tiles[e] = acc;
+      acc += (expert_counts[e] + kBM - 1) / kBM;
+    }
+    s_tiles[num_experts] = acc;
+    tile_list[0] = min(acc, capacity);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < num_experts; e += 256) {
+    const int c = expert_counts[e];
+    const int nt = (c + kBM - 1) / kBM;
+    for (int i = 0; i < nt; ++i) {
+      const int idx = s_tiles[e] + i;
+      if (idx >= capacity) break;
+      tile_list[4 + 4 * idx + 0] = e;
+      tile_list[4 + 4 * idx + 1] = s_base[e] + i * kBM;
+      tile_list[4 + 4 * idx + 2] = min(kBM, c - i * kBM);
+      tile_list[4 + 4 * idx + 3] = 0;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ host side
+static size_t stack_row_bytes(int quant, size_t K) {
+  return K / xabe_expert_quant_block_elements(quant) * xabe_expert_quant_block_bytes(quant);
+}
+
 bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int gate_q, int up_q, int down_q, bool routed) {
-  (void)k; (void)b; (void)gate_q; (void)up_q; (void)down_q; (void)routed;
-  return false;
+  const xabe_moe_geometry& g = k->g;
+  if (!k->tensor_cores || k->exact_regime || g.max_tokens < kMfmaMinTokens) return false;
+  if (!b->x_h || !b->shared_inter_h) return false;
+  if (routed && (!b->inter_h || !b->tile_list)) return false;
+  auto ok = [](int q) { return q == XABE_QUANT_Q6K || q == XABE_QUANT_Q8_0; };
+  if (!ok(gate_q) || !ok(down_q) || gate_q != up_q) return false;
+  // contraction in steps of 128 (whole Q6_K superblocks: 256); gate/up tiles 64 columns, down tiles 128
+  if (g.hidden % 256 != 0 || g.intermediate % 256 != 0) return false;
+  return true;
 }
 
-int mfma_grouped_forward_partial(const xabe_moe_kernels*, hipStream_t, xabe_moe_buffers*, xabe_quant_tensor,
-                                 xabe_quant_tensor, xabe_quant_tensor, const float*) {
-  return set_error(XABE_ERR_MMA, "matrix-core regime not built");
+template <int NM, bool ROUTED>
+static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
+  const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * 2));
+  constexpr size_t smem = (size_t)(kBM + kBR) * kLd * sizeof(_Float16) + 3 * kBM * sizeof(int);
+  auto kq6 = k_mfma_expert<kQ6K, NM, ROUTED>;
+  auto kq8 = k_mfma_expert<kQ8_0, NM, ROUTED>;
+  static bool configured = false;  // per instantiation; the attribute is per function, set once
+  if (!configured) {
+    XABE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kq6), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    XABE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kq8), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    configured = true;
+  }
+  if (quant == XABE_QUANT_Q6K) hipLaunchKernelGGL(kq6, dim3(grid), dim3(256), smem, s, a);
+  else hipLaunchKernelGGL(kq8, dim3(grid), dim3(256), smem, s, a);
+  XABE_HIP_TRY(hipGetLastError());
+  return XABE_OK;
 }
 
-int mfma_shared_expert(const xabe_moe_kernels*, hipStream_t, xabe_moe_buffers*, xabe_quant_tensor, xabe_quant_tensor,
-                       xabe_quant_tensor, const float*, float*) {
-  return set_error(XABE_ERR_MMA, "matrix-core regime not built");
+static int to_f16(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const float* x) {
+  hipLaunchKernelGGL(k_to_f16_rows, dim3((unsigned)k->g.max_tokens), dim3(256), 0, s, x, b->valid_tokens, (int)k->g.hidden,
+                     reinterpret_cast<_Float16*>(b->x_h));
+  XABE_HIP_TRY(hipGetLastError());
+  return XABE_OK;
+}
+
+int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                                 xabe_quant_tensor up, xabe_quant_tensor down, const float* x) {
+  const xabe_moe_geometry& g = k->g;
+  XABE_TRY(to_f16(k, s, b, x));
+  const int cap = (int)((b->n_tile_list - 4) / 4);
+  hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap,
+                     b->tile_list);
+  XABE_HIP_TRY(hipGetLastError());
+  MfmaArgs a;
+  memset(&a, 0, sizeof(a));
+  a.valid_tokens = b->valid_tokens;
+  a.sorted_token_ids = b->sorted_token_ids;
+  a.topk_weights = b->topk_weights;
+  a.tile_list = b->tile_list;
+  a.top_k = (int)g.experts_per_token;
+  const size_t max_mtiles = (size_t)cap;
+  // gate/up + SwiGLU -> inter_h[slot][I]
+  a.w0 = static_cast<const uint8_t*>(gate.bytes);
+  a.w1 = static_cast<const uint8_t*>(up.bytes);
+  a.expert_bytes = g.intermediate * stack_row_bytes(gate.quant, g.hidden);
+  a.a = reinterpret_cast<const _Float16*>(b->x_h);
+  a.out = b->inter_h;
+  a.K = (int)g.hidden;
+  a.n_rows = (int)g.intermediate;
+  XABE_TRY((launch_mfma<2, true>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  // down -> partial[flat][H], scaled by the routing weight
+  a.w0 = static_cast<const uint8_t*>(down.bytes);
+  a.w1 = nullptr;
+  a.expert_bytes = g.hidden * stack_row_bytes(down.quant, g.intermediate);
+  a.a = reinterpret_cast<const _Float16*>(b->inter_h);
+  a.out = b->partial;
+  a.K = (int)g.intermediate;
+  a.n_rows = (int)g.hidden;
+  XABE_TRY((launch_mfma<1, true>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
+  return XABE_OK;
+}
+
+int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                       xabe_quant_tensor up, xabe_quant_tensor down, const float* x, float* out) {
+  const xabe_moe_geometry& g = k->g;
+  XABE_TRY(to_f16(k, s, b, x));
+  MfmaArgs a;
+  memset(&a, 0, sizeof(a));
+  a.valid_tokens = b->valid_tokens;
+  a.top_k = 1;
+  const size_t max_mtiles = (g.max_tokens + kBM - 1) / kBM;
+  a.w0 = static_cast<const uint8_t*>(gate.bytes);
+  a.w1 = static_cast<const uint8_t*>(up.bytes);
+  a.a = reinterpret_cast<const _Float16*>(b->x_h);
+  a.out = b->shared_inter_h;
+  a.K = (int)g.hidden;
+  a.n_rows = (int)g.intermediate;
+  XABE_TRY((launch_mfma<2, false>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  a.w0 = static_cast<const uint8_t*>(down.bytes);
+  a.w1 = nullptr;
+  a.a = reinterpret_cast<const _Float16*>(b->shared_inter_h);
+  a.out = out;
+  a.K = (int)g.intermediate;
+  a.n_rows = (int)g.hidden;
+  XABE_TRY((launch_mfma<1, false>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
+  return XABE_OK;
 }
 
 }  // namespace xabe
