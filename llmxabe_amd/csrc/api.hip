@@ -691,7 +691,7 @@ int xabe_moe_gate_and_combine(const xabe_moe_kernels* k, void* stream, const xab
     return set_error(XABE_ERR_INVALID_ARGUMENT, "gate_and_combine: null pointer");
   XABE_TRY(require_routed(b, "gate_and_combine"));
   const xabe_moe_geometry& g = k->g;
-  dim3 grid((unsigned)g.max_tokens, (unsigned)((g.hidden + 255) / 256));
+  dim3 grid((unsigned)g.max_tokens, (unsigned)((g.hidden + 1023) / 1024));
   hipLaunchKernelGGL(k_gate_and_combine, grid, dim3(256), 0, as_stream(stream), shared_gate_inp, normed, b->partial, shexp,
                      residual, b->valid_tokens, (int)g.experts_per_token, (int)g.hidden, gate, routed, ffn_out, l_out);
   XABE_HIP_TRY(hipGetLastError());

@@ -30,6 +30,7 @@ namespace xabe {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBM = 128;          // token rows per tile
 constexpr int kBR = 128;          // weight rows per tile
@@ -54,7 +55,7 @@ struct MfmaArgs {
 };
 
 // ---- prologues: one 32-element unit of one weight row -> 32 halfs in LDS -----------------
-__device__ __forceinline__ uint4 pack8(uint32_t c0, uint32_t c1, half2v off, half2v s) {
+__device__ __forceinline__ u32x4 pack8(uint32_t c0, uint32_t c1, half2v off, half2v s) {
   // c0, c1: eight byte codes; returns eight halfs (code + 1024 - off) * s
   uint32_t p[4];
   p[0] = __builtin_amdgcn_perm(0x64646464u, c0, 0x04010400u);
@@ -68,7 +69,8 @@ __device__ __forceinline__ uint4 pack8(uint32_t c0, uint32_t c1, half2v off, hal
     v = (v + off) * s;
     o[i] = __builtin_bit_cast(uint32_t, v);
   }
-  return make_uint4(o[0], o[1], o[2], o[3]);
+  u32x4 r = {o[0], o[1], o[2], o[3]};
+  return r;
 }
 
 // Q6_K unit (half h of a superblock, l8): codes at j*32 + l8*8 + i of that half.
@@ -92,7 +94,7 @@ __device__ __forceinline__ void q6_unit_to_lds(const Q6Raw& r, int l8, _Float16*
   for (int j = 0; j < 4; ++j) {
     const _Float16 sh = (_Float16)ds[j];
     const half2v s = {sh, sh};
-    *reinterpret_cast<uint4*>(brow + j * 32 + l8 * 8) = pack8(c[0][j], c[1][j], off, s);
+    *reinterpret_cast<u32x4*>(brow + j * 32 + l8 * 8) = pack8(c[0][j], c[1][j], off, s);
   }
 }
 
@@ -103,13 +105,35 @@ __device__ __forceinline__ void q8_unit_to_lds(const Q8Raw& r, _Float16* bdst) {
   const half2v off = {(_Float16)-1152.0f, (_Float16)-1152.0f};      // 1024 (perm bias) + 128 (sign flip)
 #pragma unroll
   for (int w = 0; w < 4; ++w)
-    reinterpret_cast<uint4*>(bdst)[w] = pack8(r.q[2 * w] ^ 0x80808080u, r.q[2 * w + 1] ^ 0x80808080u, off, s);
+    reinterpret_cast<u32x4*>(bdst)[w] = pack8(r.q[2 * w] ^ 0x80808080u, r.q[2 * w + 1] ^ 0x80808080u, off, s);
 }
 
 template <int QUANT>
 struct WRaw {
   typename std::conditional<QUANT == kQ6K, Q6Raw, Q8Raw>::type u[2];
 };
+
+// Global loads of one contraction step into registers: eight 16-byte activation chunks and the
+// raw blocks of this thread's two weight-row units.
+template <int QUANT>
+__device__ __forceinline__ void load_step(int ks, const _Float16* const (&arow_ptr)[8], const uint8_t* const (&wrow)[2],
+                                          int du, u32x4 (&areg)[8], WRaw<QUANT>& wreg) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const u32x4*>(arow_ptr[i] + (size_t)ks * kBK);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    if constexpr (QUANT == kQ6K) {
+      // step ks covers half (ks & 1) of superblock ks >> 1
+      const uint8_t* p = wrow[i] + (size_t)(ks >> 1) * kQ6KBytes;
+      const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
+      q6_load(p - mis, mis, ks & 1, du, wreg.u[i]);
+    } else {
+      const uint8_t* p = wrow[i] + (size_t)(ks * 4 + du) * kQ8Bytes;
+      const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
+      q8_load(p - mis, mis, wreg.u[i]);
+    }
+  }
+}
 
 template <int QUANT, int NM, bool ROUTED>
 __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
@@ -194,32 +218,15 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    uint4 areg[8];
+    u32x4 areg[8];
     WRaw<QUANT> wreg;
-    auto load_step = [&](int ks) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const uint4*>(arow_ptr[i] + (size_t)ks * kBK);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        if constexpr (QUANT == kQ6K) {
-          // step ks covers half (ks & 1) of superblock ks >> 1
-          const uint8_t* p = wrow[i] + (size_t)(ks >> 1) * kQ6KBytes;
-          const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
-          q6_load(p - mis, mis, ks & 1, du, wreg.u[i]);
-        } else {
-          const uint8_t* p = wrow[i] + (size_t)(ks * 4 + du) * kQ8Bytes;
-          const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
-          q8_load(p - mis, mis, wreg.u[i]);
-        }
-      }
-    };
-    load_step(0);
+    load_step<QUANT>(0, arow_ptr, wrow, du, areg, wreg);
     for (int ks = 0; ks < nks; ++ks) {
       __syncthreads();  // everyone has finished reading the previous step's tiles
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int c = tid + 256 * i;
-        *reinterpret_cast<uint4*>(&sA[(c >> 4) * kLd + (c & 15) * 8]) = areg[i];
+        *reinterpret_cast<u32x4*>(&sA[(c >> 4) * kLd + (c & 15) * 8]) = areg[i];
       }
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
@@ -228,7 +235,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
         else q8_unit_to_lds(wreg.u[i], &sB[rb * kLd + du * 32]);
       }
       __syncthreads();
-      if (ks + 1 < nks) load_step(ks + 1);  // in flight while the matrix cores work
+      if (ks + 1 < nks) load_step<QUANT>(ks + 1, arow_ptr, wrow, du, areg, wreg);  // in flight while the matrix cores work
       const _Float16* pa = &sA[(wm * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
       const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
 #pragma unroll

@@ -230,7 +230,7 @@ __global__ void __launch_bounds__(256) k_moe_reduce(const float* __restrict__ pa
 // ---------------------------------------------------------------------------------
 // moe_block_gate_and_combine (crates/xabe-engine/src/block/moe.rs:424-483):
 //   g = 1/(1+expf(-(w . normed[t])));  r = sum_k partial (ascending k);
-//   ffn_out = r + shexp*g;  l_out = ffn_out + residual.   grid (max_tokens, ceil(hidden/256)).
+//   ffn_out = r + shexp*g;  l_out = ffn_out + residual.   grid (max_tokens, ceil(hidden/1024)).
 // ---------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) k_gate_and_combine(const float* __restrict__ w, const float* __restrict__ normed,
                                                            const float* __restrict__ partial, const float* __restrict__ shexp,
@@ -248,15 +248,23 @@ __global__ void __launch_bounds__(256) k_gate_and_combine(const float* __restric
   s = block_sum_256(s, scratch);
   const float g = 1.0f / (1.0f + expf(-s));
   if (threadIdx.x == 0 && blockIdx.y == 0) gate[t] = g;
-  const int j = blockIdx.y * 256 + threadIdx.x;
+  // four consecutive columns per thread (hidden is a multiple of 128)
+  const int j = (blockIdx.y * 256 + threadIdx.x) * 4;
   if (j >= hidden) return;
   const float* p = partial + (size_t)t * top_k * hidden + j;
-  float r = 0.0f;
-  for (int k = 0; k < top_k; ++k) r += p[(size_t)k * hidden];
-  const float v = r + shexp[base + j] * g;
-  routed[base + j] = r;
-  ffn_out[base + j] = v;
-  l_out[base + j] = v + residual[base + j];
+  float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k = 0; k < top_k; ++k) {
+    const float4 v = *reinterpret_cast<const float4*>(p + (size_t)k * hidden);
+    r.x += v.x; r.y += v.y; r.z += v.z; r.w += v.w;
+  }
+  const float4 sh = *reinterpret_cast<const float4*>(shexp + base + j);
+  const float4 rs = *reinterpret_cast<const float4*>(residual + base + j);
+  float4 v, lo;
+  v.x = r.x + sh.x * g; v.y = r.y + sh.y * g; v.z = r.z + sh.z * g; v.w = r.w + sh.w * g;
+  lo.x = v.x + rs.x; lo.y = v.y + rs.y; lo.z = v.z + rs.z; lo.w = v.w + rs.w;
+  *reinterpret_cast<float4*>(routed + base + j) = r;
+  *reinterpret_cast<float4*>(ffn_out + base + j) = v;
+  *reinterpret_cast<float4*>(l_out + base + j) = lo;
 }
 
 // dense_ffn_add_residual (crates/xabe-engine/src/block/dense_ffn.rs:1149-1175)
