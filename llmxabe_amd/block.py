@@ -49,7 +49,10 @@ class MoeBlock:
 
     def __del__(self):
         if getattr(self, "_h", None):
-            _ffi.lib().xabe_moe_block_free(self._h)
+            try:
+                _ffi.lib().xabe_moe_block_free(self._h)
+            except Exception:  # interpreter shutdown
+                pass
             self._h = None
 
     def geometry(self) -> MoeGeometry: return self._geometry
@@ -57,6 +60,7 @@ class MoeBlock:
     def disable_tensor_cores(self): check(_ffi.lib().xabe_moe_block_disable_tensor_cores(self._h))
     def set_exact_decode_regime(self, on: bool): check(_ffi.lib().xabe_moe_block_set_exact_decode_regime(self._h, int(on)))
     def tensor_cores_enabled(self) -> bool: return bool(_ffi.lib().xabe_moe_block_tensor_cores_enabled(self._h))
+    def set_fused_decode(self, on: bool): check(_ffi.lib().xabe_moe_block_set_fused_decode(self._h, int(on)))
 
     def publish_tokens(self, tokens: int):
         check(_ffi.lib().xabe_moe_block_publish_tokens(self._h, _stream(), tokens))
@@ -102,7 +106,10 @@ class DenseFfnBlock:
 
     def __del__(self):
         if getattr(self, "_h", None):
-            _ffi.lib().xabe_dense_ffn_block_free(self._h)
+            try:
+                _ffi.lib().xabe_dense_ffn_block_free(self._h)
+            except Exception:  # interpreter shutdown
+                pass
             self._h = None
 
     def disable_tensor_cores(self): check(_ffi.lib().xabe_dense_ffn_block_disable_tensor_cores(self._h))

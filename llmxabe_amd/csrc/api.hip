@@ -121,19 +121,23 @@ static void launch_shape(Shape shape, Mode mode, dim3 grid, hipStream_t s, const
   }
 }
 
-// `units`: grid.x work units (pairs, dispatch blocks, token chunks); `live_units`: how many
+int pick_tile_rows(const xabe_moe_kernels* k, size_t live_units, int n_rows, int rps) {
+  // aim for ~12 wavefronts per CU across the launch
+  const size_t items = std::max<size_t>(1, live_units) * (size_t)n_rows / rps;
+  const size_t target_waves = (size_t)k->num_cus * 12;
+  const size_t per_wave = (items + target_waves - 1) / target_waves;
+  size_t pw = 1;
+  while (pw < per_wave && pw < 16) pw <<= 1;
+  return (int)(pw * kWavesPerWg * rps);
+}
+
+// `units`: grid.y work units (pairs, dispatch blocks, token chunks); `live_units`: how many
 // of them a typical step actually uses, for sizing the row tile.
 static int launch_expert(const xabe_moe_kernels* k, Mode mode, int quant, int nm, ExpertArgs a, size_t units,
                          size_t live_units, hipStream_t s) {
   const Shape shape = shape_for((size_t)a.K);
   const int rps = rows_per_step(shape);
-  // rows per workgroup: aim for ~12 wavefronts per CU across the launch
-  const size_t items = std::max<size_t>(1, live_units) * (size_t)a.n_rows / rps;
-  const size_t target_waves = (size_t)k->num_cus * 12;
-  size_t per_wave = (items + target_waves - 1) / target_waves;
-  size_t pw = 1;
-  while (pw < per_wave && pw < 16) pw <<= 1;
-  a.tile_rows = (int)(pw * kWavesPerWg * rps);
+  a.tile_rows = pick_tile_rows(k, live_units, a.n_rows, rps);
   const unsigned tiles = (unsigned)((a.n_rows + a.tile_rows - 1) / a.tile_rows);
   if (tiles > 65535) return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "row-tile count %u exceeds the grid.y limit", tiles);
   dim3 grid(tiles, (unsigned)units);  // x = row tile (fast), y = unit
@@ -417,6 +421,7 @@ int xabe_moe_route(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b,
   const xabe_moe_geometry& g = k->g;
   if (g.num_experts > kRouteMaxExperts)
     return bad_geometry(g, "the routing wavefront holds 8 experts per lane, so at most 512 experts");
+  if (g.experts_per_token > 64) return bad_geometry(g, "the routing wavefront keeps one selection per lane, so at most top-64");
   XABE_TRY(check_len("logits", g.max_tokens * g.num_experts, logits_len));
   const unsigned grid = (unsigned)((g.max_tokens + 3) / 4);
   const size_t smem = 4 * g.num_experts * sizeof(float);
@@ -619,9 +624,20 @@ int xabe_moe_grouped_forward_partial_with_shared(const xabe_moe_kernels* k, void
   XABE_TRY(check_shared_stacks(k, shared_gate, shared_up, shared_down));
   XABE_TRY(check_len("hidden_states", g.max_tokens * g.hidden, hidden_states_len));
   XABE_TRY(check_len("out", g.max_tokens * g.hidden, out_len));
-  // Same bodies as the separate entry points, so the outputs are bit-identical to them.
-  XABE_TRY(routed_fp32(k, as_stream(stream), b, gate, up, down, hidden_states));
-  XABE_TRY(shared_fp32(k, as_stream(stream), b, shared_gate, shared_up, shared_down, hidden_states, out));
+  // The shared expert's units ride the routed grid: two launches instead of four.  Same bodies as the
+  // separate entry points, so the outputs are bit-identical to them.
+  {
+    const size_t expert_elems = g.intermediate * g.hidden;
+    hipStream_t s = as_stream(stream);
+    const size_t gate_eb = expert_elems / xabe_expert_quant_block_elements(gate.quant) * xabe_expert_quant_block_bytes(gate.quant);
+    const size_t down_eb = expert_elems / xabe_expert_quant_block_elements(down.quant) * xabe_expert_quant_block_bytes(down.quant);
+    XABE_TRY(launch_flat_with_shared(k, s, b, 2, gate.quant, shared_gate.quant, gate.bytes, up.bytes, gate_eb, hidden_states,
+                                     b->inter, shared_gate.bytes, shared_up.bytes, hidden_states, b->shared_inter,
+                                     (int)g.hidden, (int)g.intermediate));
+    XABE_TRY(launch_flat_with_shared(k, s, b, 1, down.quant, shared_down.quant, down.bytes, nullptr, down_eb, b->inter,
+                                     b->partial, shared_down.bytes, nullptr, b->shared_inter, out, (int)g.intermediate,
+                                     (int)g.hidden));
+  }
   *fused = 1;
   return XABE_OK;
 }
@@ -649,6 +665,7 @@ int xabe_rms_norm(void* stream, const float* x, size_t x_len, const float* weigh
   XABE_TRY(check_len("weight", width, weight_len));
   XABE_TRY(check_len("out", rows * width, out_len));
   if (rows == 0 || width == 0) return XABE_OK;
+  if (width % 4 != 0) return set_error(XABE_ERR_INVALID_ARGUMENT, "rms_norm: width %zu is not a multiple of 4", width);
   hipLaunchKernelGGL(k_rms_norm_rows, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), x, weight, out, (int)width, eps);
   XABE_HIP_TRY(hipGetLastError());
   return XABE_OK;

@@ -14,6 +14,7 @@ struct xabe_moe_block {
   float eps;
   float *normed, *logits, *routed, *shexp, *gate;
   size_t n_act, n_logits;
+  int fused_decode;  // decode widths: the regrouped three-launch block where the shape allows
 };
 
 static int block_alloc(float** p, size_t n, hipStream_t s) {
@@ -28,6 +29,7 @@ int xabe_moe_block_new(const xabe_moe_geometry* geometry, float eps, void* strea
   memset(blk, 0, sizeof(*blk));
   blk->g = *geometry;
   blk->eps = eps;
+  blk->fused_decode = 1;
   int st = xabe_moe_kernels_new(geometry, &blk->moe);
   if (st == XABE_OK) st = xabe_moe_buffers_new(blk->moe, stream, &blk->buffers);
   blk->n_act = geometry->max_tokens * geometry->hidden;
@@ -78,6 +80,11 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
   XABE_TRY(blk_check_len("l_out", blk->n_act, l_out_len));
   XABE_TRY(xabe_moe_block_publish_tokens(blk, stream, tokens));
 
+  // decode widths, model shapes: the eight steps below regrouped into three launches, same arithmetic
+  if (blk->fused_decode && !blk->moe->exact_regime && decode_block_supported(blk->moe, blk->buffers, w))
+    return launch_decode_block(blk->moe, as_stream(stream), blk->buffers, w, residual, logit_bias, blk->eps, blk->normed,
+                               blk->logits, blk->shexp, blk->gate, blk->routed, ffn_out, l_out);
+
   // 1. post-mixer RMSNorm over every row of the buffer
   XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
                          g.hidden, blk->eps));
@@ -119,6 +126,11 @@ int xabe_moe_block_disable_tensor_cores(xabe_moe_block* blk) {
 int xabe_moe_block_set_exact_decode_regime(xabe_moe_block* blk, int on) {
   if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_exact_decode_regime: null handle");
   return xabe_moe_kernels_set_exact_decode_regime(blk->moe, on);
+}
+int xabe_moe_block_set_fused_decode(xabe_moe_block* blk, int on) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_fused_decode: null handle");
+  blk->fused_decode = on != 0;
+  return XABE_OK;
 }
 int xabe_moe_block_tensor_cores_enabled(const xabe_moe_block* blk) {
   return blk ? xabe_moe_kernels_tensor_cores_enabled(blk->moe) : 0;

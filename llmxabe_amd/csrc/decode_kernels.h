@@ -71,34 +71,74 @@ __device__ __forceinline__ int lane_koff(const LaneGeom& g, int k) {
   return ((g.lane % (64 / RPS)) + k * 64) * 32;
 }
 
-template <int QUANT>
-__device__ __forceinline__ void load_x(const float* __restrict__ xrow, int koff, bool active, const LaneGeom& g,
-                                       float (&x)[32], float (&xs)[4]) {
-  if (QUANT == kQ6K) {
+// How a kernel obtains its activations and publishes its outputs.
+//   kXPlain: read fp32 rows as they are.
+//   kXNorm:  RMS-normalise on load, (x * inv_rms) * norm_weight -- the same two products, in the same
+//            order, as the stand-alone RMSNorm kernel, so the values are bit-identical to its output.
+//   kXCoherent: the rows were written earlier in the SAME launch by other workgroups; read them with
+//            agent-scope loads (sc1) so another XCD's writes are visible without a cache flush.
+constexpr int kXPlain = 0, kXNorm = 1, kXCoherent = 2;
+// kOPlain: ordinary stores.  kOCoherent: agent-scope stores (written through to the coherence point).
+constexpr int kOPlain = 0, kOCoherent = 1;
+
+struct XNorm {
+  float inv;              // 1 / sqrt(mean(x^2) + eps) of this token
+  const float* weight;    // norm weight, indexed like the row
+};
+
+__device__ __forceinline__ float2 load2_coherent(const float* p) {
+  const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+  return make_float2(__builtin_bit_cast(float, (uint32_t)v), __builtin_bit_cast(float, (uint32_t)(v >> 32)));
+}
+__device__ __forceinline__ void store_coherent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Eight consecutive activations starting at xrow + off (off a multiple of 4).
+template <int XMODE>
+__device__ __forceinline__ void load8(const float* __restrict__ xrow, int off, const XNorm& nm, float (&v)[8]) {
+  if constexpr (XMODE == kXCoherent) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-      if (active) {
-        const float4* p = reinterpret_cast<const float4*>(xrow + koff + g.half * 128 + j * 32 + g.l8 * 8);
-        a = p[0];
-        b = p[1];
-      }
-      x[j * 8 + 0] = a.x; x[j * 8 + 1] = a.y; x[j * 8 + 2] = a.z; x[j * 8 + 3] = a.w;
-      x[j * 8 + 4] = b.x; x[j * 8 + 5] = b.y; x[j * 8 + 6] = b.z; x[j * 8 + 7] = b.w;
-      float s = 0.0f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) s += x[j * 8 + i];
-      xs[j] = -32.0f * s;
+    for (int i = 0; i < 4; ++i) {
+      const float2 a = load2_coherent(xrow + off + 2 * i);
+      v[2 * i] = a.x;
+      v[2 * i + 1] = a.y;
     }
   } else {
+    const float4 a = reinterpret_cast<const float4*>(xrow + off)[0];
+    const float4 b = reinterpret_cast<const float4*>(xrow + off)[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    if constexpr (XMODE == kXNorm) {
+      const float4 wa = reinterpret_cast<const float4*>(nm.weight + off)[0];
+      const float4 wb = reinterpret_cast<const float4*>(nm.weight + off)[1];
+      const float w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (active) a = reinterpret_cast<const float4*>(xrow + koff)[j];
-      x[j * 4 + 0] = a.x; x[j * 4 + 1] = a.y; x[j * 4 + 2] = a.z; x[j * 4 + 3] = a.w;
+      for (int i = 0; i < 8; ++i) v[i] = v[i] * nm.inv * w[i];
     }
+  }
+}
+
+template <int QUANT, int XMODE = kXPlain>
+__device__ __forceinline__ void load_x(const float* __restrict__ xrow, int koff, bool active, const LaneGeom& g,
+                                       float (&x)[32], float (&xs)[4], const XNorm& nm = XNorm{1.0f, nullptr}) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) xs[j] = 0.0f;
+  for (int j = 0; j < 4; ++j) {
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // Q6_K: run j of the lane's superblock unit; Q8_0 / fp32: the j-th eight of 32 consecutive elements
+    const int off = QUANT == kQ6K ? koff + g.half * 128 + j * 32 + g.l8 * 8 : koff + j * 8;
+    if (active) load8<XMODE>(xrow, off, nm, v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[j * 8 + i] = v[i];
+    if (QUANT == kQ6K) {
+      float s = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s += v[i];
+      xs[j] = -32.0f * s;
+    } else {
+      xs[j] = 0.0f;
+    }
   }
 }
 
@@ -151,11 +191,11 @@ __device__ __forceinline__ void accum(const typename Fmt<QUANT>::Raw& r, const L
 // are split over the workgroup's four wavefronts.  KS > 0: steps per row, activations
 // in registers.  KS == 0: steps from K at run time, activations re-read per step.
 // ---------------------------------------------------------------------------------
-template <int QUANT, int KS, int RPS, int TC, int NM>
+template <int QUANT, int KS, int RPS, int TC, int NM, int XMODE = kXPlain, int OMODE = kOPlain>
 __device__ __forceinline__ void matvec_rows(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, int K,
                                             int n_rows, int tile0, int tile_rows,
                                             const float* const (&xrow)[TC], float* const (&out)[TC],
-                                            const float (&scale)[TC]) {
+                                            const float (&scale)[TC], const XNorm* norm = nullptr) {
   using F = Fmt<QUANT>;
   using Raw = typename F::Raw;
   constexpr int G = 64 / RPS;
@@ -174,7 +214,8 @@ __device__ __forceinline__ void matvec_rows(const uint8_t* __restrict__ w0, cons
       const int koff = lane_koff<QUANT, RPS>(g, k);
       active[k] = koff < K;
 #pragma unroll
-      for (int t = 0; t < TC; ++t) load_x<QUANT>(xrow[t], koff, active[k], g, x[k][t], xs[k][t]);
+      for (int t = 0; t < TC; ++t)
+        load_x<QUANT, XMODE>(xrow[t], koff, active[k], g, x[k][t], xs[k][t], XMODE == kXNorm ? norm[t] : XNorm{1.0f, nullptr});
     }
     auto load_item = [&](int row0, Raw (&r)[NM][KS]) {
 #pragma unroll
@@ -200,7 +241,8 @@ __device__ __forceinline__ void matvec_rows(const uint8_t* __restrict__ w0, cons
 #pragma unroll
         for (int t = 0; t < TC; ++t) {
           const float v = NM == 2 ? silu_f(tot[0][t]) * tot[NM - 1][t] : scale[t] * tot[0][t];
-          out[t][row] = v;
+          if constexpr (OMODE == kOCoherent) store_coherent(&out[t][row], v);
+          else out[t][row] = v;
         }
       }
     };
@@ -238,7 +280,8 @@ __device__ __forceinline__ void matvec_rows(const uint8_t* __restrict__ w0, cons
         float x[TC][32];
         float xs[TC][4];
 #pragma unroll
-        for (int t = 0; t < TC; ++t) load_x<QUANT>(xrow[t], koff, act, g, x[t], xs[t]);
+        for (int t = 0; t < TC; ++t)
+          load_x<QUANT, XMODE>(xrow[t], koff, act, g, x[t], xs[t], XMODE == kXNorm ? norm[t] : XNorm{1.0f, nullptr});
         const size_t off = (size_t)row0 * row_bytes + (size_t)k * F::kChunkBytes;
         Raw r0;
         load_raw<QUANT>(w0 + off, act, g, r0);
@@ -257,7 +300,8 @@ __device__ __forceinline__ void matvec_rows(const uint8_t* __restrict__ w0, cons
 #pragma unroll
         for (int t = 0; t < TC; ++t) {
           const float v = NM == 2 ? silu_f(tot[0][t]) * tot[NM - 1][t] : scale[t] * tot[0][t];
-          out[t][row0] = v;
+          if constexpr (OMODE == kOCoherent) store_coherent(&out[t][row0], v);
+          else out[t][row0] = v;
         }
       }
     }
@@ -290,8 +334,7 @@ struct ExpertArgs {
 // (token, k) pair read straight from topk_ids; no dispatch table
 // (crates/xabe-cuda/src/kernels/moe.rs:2525-2634, :3066-3124).
 template <int QUANT, int KS, int RPS, int NM>
-__global__ void __launch_bounds__(256) k_expert_flat(ExpertArgs a) {
-  const int p = blockIdx.y;
+__device__ __forceinline__ void flat_body(const ExpertArgs& a, int p, int tile) {
   const int valid = *a.valid_tokens;
   if (p >= valid * a.top_k) return;
   const int e = a.topk_ids[p];
@@ -301,7 +344,12 @@ __global__ void __launch_bounds__(256) k_expert_flat(ExpertArgs a) {
   const float* const xr[1] = {a.x + (size_t)(NM == 2 ? p / a.top_k : p) * a.K};
   float* const o[1] = {a.out + (size_t)p * a.n_rows};
   const float sc[1] = {NM == 2 ? 1.0f : a.topk_weights[p]};
-  matvec_rows<QUANT, KS, RPS, 1, NM>(w0, w1, a.K, a.n_rows, blockIdx.x * a.tile_rows, a.tile_rows, xr, o, sc);
+  matvec_rows<QUANT, KS, RPS, 1, NM>(w0, w1, a.K, a.n_rows, tile * a.tile_rows, a.tile_rows, xr, o, sc);
+}
+
+template <int QUANT, int KS, int RPS, int NM>
+__global__ void __launch_bounds__(256) k_expert_flat(ExpertArgs a) {
+  flat_body<QUANT, KS, RPS, NM>(a, blockIdx.y, blockIdx.x);
 }
 
 // Dispatch-table regime: one work unit per dispatch block; the block's live slots all
@@ -342,21 +390,42 @@ __global__ void __launch_bounds__(256) k_expert_block(ExpertArgs a) {
 // Shared expert / dense MLP: every live token, no indirection, no routing weight
 // (crates/xabe-cuda/src/kernels/moe.rs:3425-3725, :4082-4227).  One work unit per chunk of two tokens.
 template <int QUANT, int KS, int RPS, int NM>
-__global__ void __launch_bounds__(256) k_expert_shared(ExpertArgs a) {
-  const int t0 = blockIdx.y * 2;
+__device__ __forceinline__ void shared_body(const ExpertArgs& a, int chunk, int tile) {
+  const int t0 = chunk * 2;
   const int valid = *a.valid_tokens;
   if (t0 >= valid) return;
   if (t0 + 1 < valid) {
     const float* const xr[2] = {a.x + (size_t)t0 * a.K, a.x + (size_t)(t0 + 1) * a.K};
     float* const o[2] = {a.out + (size_t)t0 * a.n_rows, a.out + (size_t)(t0 + 1) * a.n_rows};
     const float sc[2] = {1.0f, 1.0f};
-    matvec_rows<QUANT, KS, RPS, 2, NM>(a.w0, a.w1, a.K, a.n_rows, blockIdx.x * a.tile_rows, a.tile_rows, xr, o, sc);
+    matvec_rows<QUANT, KS, RPS, 2, NM>(a.w0, a.w1, a.K, a.n_rows, tile * a.tile_rows, a.tile_rows, xr, o, sc);
   } else {
     const float* const xr[1] = {a.x + (size_t)t0 * a.K};
     float* const o[1] = {a.out + (size_t)t0 * a.n_rows};
     const float sc[1] = {1.0f};
-    matvec_rows<QUANT, KS, RPS, 1, NM>(a.w0, a.w1, a.K, a.n_rows, blockIdx.x * a.tile_rows, a.tile_rows, xr, o, sc);
+    matvec_rows<QUANT, KS, RPS, 1, NM>(a.w0, a.w1, a.K, a.n_rows, tile * a.tile_rows, a.tile_rows, xr, o, sc);
   }
+}
+
+template <int QUANT, int KS, int RPS, int NM>
+__global__ void __launch_bounds__(256) k_expert_shared(ExpertArgs a) {
+  shared_body<QUANT, KS, RPS, NM>(a, blockIdx.y, blockIdx.x);
+}
+
+// The shared expert's work units appended to the routed grid (blockIdx.y >= routed_units), each
+// unit running the body its separate launch runs, so every output is bit-identical to the
+// four-launch form (crates/xabe-cuda/src/kernels/moe.rs:3727-4032).
+struct FusedArgs {
+  ExpertArgs routed;
+  ExpertArgs shared;
+  int routed_units;
+};
+
+template <int RQ, int SQ, int KS, int RPS, int NM>
+__global__ void __launch_bounds__(256) k_expert_flat_with_shared(FusedArgs a) {
+  const int unit = blockIdx.y;
+  if (unit < a.routed_units) flat_body<RQ, KS, RPS, NM>(a.routed, unit, blockIdx.x);
+  else shared_body<SQ, KS, RPS, NM>(a.shared, unit - a.routed_units, blockIdx.x);
 }
 
 }  // namespace xabe

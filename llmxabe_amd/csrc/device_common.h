@@ -56,9 +56,80 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+// Wavefront max / min over all 64 lanes (order-free, exact): DPP within 16-lane rows, then the four row
+// results through scalar broadcasts.  Every lane receives the result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
 __device__ __forceinline__ float wave_max(float v) {
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  v = fmaxf(v, dpp_f<0x4E>(v));
+  v = fmaxf(v, dpp_f<0x141>(v));
+  v = fmaxf(v, dpp_f<0x140>(v));
+  return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
+}
+__device__ __forceinline__ int wave_max_i(int v) {
+  v = max(v, dpp_i<0xB1>(v));
+  v = max(v, dpp_i<0x4E>(v));
+  v = max(v, dpp_i<0x141>(v));
+  v = max(v, dpp_i<0x140>(v));
+  const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+  const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+  return max(max(a, b), max(c, d));
+}
+__device__ __forceinline__ int wave_min_i(int v) {
+  v = min(v, dpp_i<0xB1>(v));
+  v = min(v, dpp_i<0x4E>(v));
+  v = min(v, dpp_i<0x141>(v));
+  v = min(v, dpp_i<0x140>(v));
+  const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+  const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+  return min(min(a, b), min(c, d));
+}
+
+// 1 / sqrt(mean(x^2) + eps) of one row, computed by one wavefront in a fixed order: lane L folds
+// elements 32L..32L+31 of every 2048-element chunk sequentially, then the wavefront tree.  Every kernel
+// that needs the RMS scale of a token goes through rms_fold / rms_finish, so they all see the same bits.
+struct RmsRaw {
+  float4 q[8];  // the lane's 32 elements of one chunk (zeros past the end of the row: fma(0, 0, s) == s)
+};
+
+__device__ __forceinline__ void rms_load(const float* __restrict__ x, int chunk0, int width, RmsRaw& r) {
+  const int base = chunk0 + (int)__lane_id() * 32;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)  // width is a multiple of 4
+    r.q[i] = base + 4 * i < width ? reinterpret_cast<const float4*>(x + base)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+__device__ __forceinline__ float rms_fold(const RmsRaw& r, float s) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    s = __builtin_fmaf(r.q[i].x, r.q[i].x, s);
+    s = __builtin_fmaf(r.q[i].y, r.q[i].y, s);
+    s = __builtin_fmaf(r.q[i].z, r.q[i].z, s);
+    s = __builtin_fmaf(r.q[i].w, r.q[i].w, s);
+  }
+  return s;
+}
+
+__device__ __forceinline__ float rms_finish(float lane_sum, int width, float eps) {
+  const float ss = group_sum<64>(lane_sum);
+  return 1.0f / sqrtf(ss / (float)width + eps);
+}
+
+__device__ __forceinline__ float row_inv_rms(const float* __restrict__ x, int width, float eps) {
+  float s = 0.0f;
+  for (int c = 0; c < width; c += 2048) {
+    RmsRaw r;
+    rms_load(x, c, width, r);
+    s = rms_fold(r, s);
+  }
+  return rms_finish(s, width, eps);
 }
 
 // ---------------------------------------------------------------------------------

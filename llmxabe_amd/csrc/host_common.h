@@ -46,6 +46,20 @@ struct xabe_moe_kernels;
 struct xabe_moe_buffers;
 
 namespace xabe {
+// decode-width fusions (fused.hip).  `quant` < 0 means plain fp32 rows.
+int launch_flat_with_shared(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, int nm, int routed_quant,
+                            int shared_quant, const void* rw0, const void* rw1, size_t expert_bytes, const float* rx,
+                            float* rout, const void* sw0, const void* sw1, const float* sx, float* sout, int K,
+                            int n_rows);
+// rows per workgroup for a launch with `live_units` busy work units
+int pick_tile_rows(const xabe_moe_kernels* k, size_t live_units, int n_rows, int rows_per_step);
+
+// the decode-width block in three launches (decode_block.hip)
+bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, const xabe_moe_layer_weights* w);
+int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, const xabe_moe_layer_weights* w,
+                        const float* residual, const float* logit_bias, float eps, float* normed, float* logits,
+                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out);
+
 // matrix-core regime (mfma.hip)
 bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int gate_q, int up_q, int down_q, bool routed);
 int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,

@@ -1,0 +1,136 @@
+// Routing of one token on one wavefront, shared by the stand-alone route kernel and the
+// single-launch router + route kernel (so both give the same bits).
+#pragma once
+
+#include "device_common.h"
+
+#ifndef XABE_ROUTE_TRACE
+#define XABE_ROUTE_TRACE(slot) do { } while (0)
+#endif
+
+namespace xabe {
+
+constexpr int kRouteMaxPerLane = 8;  // 64 lanes x 8 = 512 experts
+
+// Routes one token on one wavefront, in two parts so that a caller can put other loads between them.
+// route_load: the token's logits `lg` into registers, expert i*64+lane in l[i]; `bias` (may be null) is
+// added first and the sums are written back to `lg_out`.  route_compute: `e_all` is num_experts floats of
+// LDS private to this wavefront; lanes 0..top_k-1 return the k-th selection in (sel_i, sel_w).
+// PER: experts held per lane, num_experts <= 64 * PER.
+//
+// The arithmetic is the reference's, operation for operation: e = (float)exp((double)(l - max)), the
+// sum of e in index order, p = e / sum, the k largest p with the lower index winning a tie, weights
+// p / (sum of the selected p in selection order).
+template <int PER, bool COHERENT = false>
+__device__ __forceinline__ void route_load(const float* lg, int num_experts, const float* __restrict__ bias,
+                                           float* lg_out, float (&l)[PER]) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int idx = i * 64 + lane;
+    l[i] = -INFINITY;
+    if (idx < num_experts)
+      l[i] = COHERENT ? __hip_atomic_load(lg + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[idx];
+    if (bias && idx < num_experts) {
+      l[i] += bias[idx];
+      lg_out[idx] = l[i];
+    }
+  }
+}
+
+template <int PER>
+__device__ __forceinline__ void route_compute(const float (&l)[PER], int num_experts, int top_k, float* e_all,
+                                              int& sel_i, float& sel_w) {
+  const int lane = threadIdx.x & 63;
+  float m = l[0];
+#pragma unroll
+  for (int i = 1; i < PER; ++i) m = fmaxf(m, l[i]);
+  m = wave_max(m);
+  XABE_ROUTE_TRACE(1);
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int idx = i * 64 + lane;
+    if (idx < num_experts) e_all[idx] = (float)exp((double)(l[i] - m));
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  XABE_ROUTE_TRACE(2);
+  // sequential sum in index order on lane 0 alone (a 16-byte LDS read that all 64 lanes aim at one
+  // address is serialised lane by lane), 32 values per batch so that the reads are in flight together and
+  // only the additions form the dependent chain
+  float sum = -0.0f;
+  if (lane == 0) {
+    const int n32 = num_experts & ~31;
+    for (int i = 0; i < n32; i += 32) {
+      float4 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const float4*>(e_all + i + 4 * j);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        sum += v[j].x;
+        sum += v[j].y;
+        sum += v[j].z;
+        sum += v[j].w;
+      }
+    }
+    for (int i = n32; i < num_experts; ++i) sum += e_all[i];
+  }
+  sum = lane_bcast(sum, 0);
+  XABE_ROUTE_TRACE(3);
+  // p >= +0, so the bit patterns order like the values and the selection runs on integers (one DPP
+  // max per reduction step, no NaN canonicalisation); kTaken marks entries that are out of the running
+  constexpr int kTaken = -1;
+  int p[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int idx = i * 64 + lane;
+    p[i] = idx < num_experts ? __builtin_bit_cast(int, e_all[idx] / sum) : kTaken;
+  }
+  // top-k: each round takes the largest p not yet taken, the lowest index among equals
+  int sel_bits = 0;
+  sel_i = 0;
+  for (int k = 0; k < top_k; ++k) {
+    int bp = p[0];
+#pragma unroll
+    for (int i = 1; i < PER; ++i) bp = max(bp, p[i]);
+    const int best = wave_max_i(bp);
+    int li = 0x7fffffff;
+#pragma unroll
+    for (int i = PER - 1; i >= 0; --i)
+      if (p[i] == best) li = i * 64 + lane;  // descending i: the lowest index of this lane wins
+    const unsigned long long holders = __builtin_amdgcn_ballot_w64(li != 0x7fffffff);
+    int bi;
+    if (__builtin_popcountll(holders) == 1) bi = __builtin_amdgcn_readlane(li, __builtin_ctzll(holders));
+    else bi = wave_min_i(li);
+    if (lane == k) { sel_bits = best; sel_i = bi; }
+    if ((bi & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < PER; ++i)
+        if (i == (bi >> 6)) p[i] = kTaken;
+    }
+  }
+  const float sel_p = __builtin_bit_cast(float, sel_bits);
+  XABE_ROUTE_TRACE(4);
+  // sum of the selected probabilities in selection order
+  float ssum = -0.0f;
+  for (int k = 0; k < top_k; ++k) ssum += lane_bcast(sel_p, k);
+  sel_w = ssum > 0.0f ? sel_p / ssum : 1.0f / (float)top_k;
+}
+
+template <bool COHERENT = false>
+__device__ __forceinline__ void route_one_token(const float* lg, int num_experts, int top_k, float* e_all,
+                                                int& sel_i, float& sel_w, const float* __restrict__ bias = nullptr,
+                                                float* lg_out = nullptr) {
+  if (num_experts <= 256) {
+    float l[4];
+    route_load<4, COHERENT>(lg, num_experts, bias, lg_out, l);
+    route_compute<4>(l, num_experts, top_k, e_all, sel_i, sel_w);
+  } else {
+    float l[kRouteMaxPerLane];
+    route_load<kRouteMaxPerLane, COHERENT>(lg, num_experts, bias, lg_out, l);
+    route_compute<kRouteMaxPerLane>(l, num_experts, top_k, e_all, sel_i, sel_w);
+  }
+}
+
+}  // namespace xabe

@@ -3,6 +3,7 @@
 #pragma once
 
 #include "device_common.h"
+#include "route_device.h"
 
 namespace xabe {
 
@@ -24,30 +25,11 @@ __device__ __forceinline__ float block_sum_256(float v, float* scratch) {
 // ---------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__ x, const float* __restrict__ w,
                                                         float* __restrict__ out, int width, float eps) {
-  __shared__ float scratch[4];
   const float* xr = x + (size_t)blockIdx.x * width;
   float* o = out + (size_t)blockIdx.x * width;
-  float s = 0.0f;
-  for (int j = threadIdx.x; j < width; j += 256) {
-    const float v = xr[j];
-    s = __builtin_fmaf(v, v, s);
-  }
-  const float ss = block_sum_256(s, scratch);
-  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  const float inv = row_inv_rms(xr, width, eps);  // each wavefront computes the same scale
   for (int j = threadIdx.x; j < width; j += 256) o[j] = xr[j] * inv * w[j];
 }
-
-// ---------------------------------------------------------------------------------
-// route (crates/xabe-cuda/src/kernels/moe.rs:1852-2036; CPU: crates/xabe-kernels/src/moe/router.rs:32-76).
-// One wavefront per token, four tokens per workgroup.  The arithmetic is the CPU
-// reference's, operation for operation, so the selected ids are the ones route_token
-// returns for these logits: max (order-free), e = exp(l - max), the sum of e taken
-// sequentially in index order, p = e / sum, top-k by (p descending, index ascending),
-// weights p / (sum of the selected p in selection order).
-// exp is evaluated in double and rounded once, which is the correctly rounded fp32 exp
-// except on a ~2^-29 fraction of inputs.
-// ---------------------------------------------------------------------------------
-constexpr int kRouteMaxPerLane = 8;  // 64 lanes x 8 = 512 experts
 
 __global__ void __launch_bounds__(256) k_route(const float* __restrict__ logits, const int* __restrict__ valid_tokens,
                                                 int num_experts, int top_k, int* __restrict__ topk_ids,
@@ -56,65 +38,13 @@ __global__ void __launch_bounds__(256) k_route(const float* __restrict__ logits,
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= *valid_tokens) return;
-  float* e_all = route_smem + (size_t)wave * num_experts;
-  const float* lg = logits + (size_t)t * num_experts;
-  const int per = (num_experts + 63) >> 6;
-
-  float l[kRouteMaxPerLane];
-  float m = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < kRouteMaxPerLane; ++i) {
-    const int idx = i * 64 + lane;
-    l[i] = (i < per && idx < num_experts) ? lg[idx] : -INFINITY;
-    m = fmaxf(m, l[i]);
-  }
-  m = wave_max(m);
-#pragma unroll
-  for (int i = 0; i < kRouteMaxPerLane; ++i) {
-    const int idx = i * 64 + lane;
-    if (i < per && idx < num_experts) e_all[idx] = (float)exp((double)(l[i] - m));
-  }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  // sequential sum, every lane redundantly (LDS broadcast reads)
-  float sum = -0.0f;
-  for (int i = 0; i < num_experts; ++i) sum += e_all[i];
-  float p[kRouteMaxPerLane];
-#pragma unroll
-  for (int i = 0; i < kRouteMaxPerLane; ++i) {
-    const int idx = i * 64 + lane;
-    p[i] = (i < per && idx < num_experts) ? e_all[idx] / sum : -1.0f;  // -1: never selected
-  }
-  // top-k: each round takes the (p max, idx min) over everything not yet taken
-  float sel_p = 0.0f;  // lane k keeps the k-th selected probability
-  int sel_i = 0;
-  for (int k = 0; k < top_k; ++k) {
-    float bp = -1.0f;
-    int bi = 0x7fffffff;
-#pragma unroll
-    for (int i = 0; i < kRouteMaxPerLane; ++i) {
-      const int idx = i * 64 + lane;
-      if (p[i] > bp) { bp = p[i]; bi = idx; }  // ascending idx within a lane, strict > keeps the lower
-    }
-    for (int off = 32; off > 0; off >>= 1) {
-      const float op = __shfl_xor(bp, off, 64);
-      const int oi = __shfl_xor(bi, off, 64);
-      if (op > bp || (op == bp && oi < bi)) { bp = op; bi = oi; }
-    }
-    if (lane == k) { sel_p = bp; sel_i = bi; }
-    if ((bi & 63) == lane) {
-#pragma unroll
-      for (int i = 0; i < kRouteMaxPerLane; ++i)
-        if (i == (bi >> 6)) p[i] = -1.0f;
-    }
-  }
-  // selected sum in selection order
-  float ssum = -0.0f;
-  for (int k = 0; k < top_k; ++k) ssum += __shfl(sel_p, k, 64);
+  int sel_i;
+  float sel_w;
+  route_one_token(logits + (size_t)t * num_experts, num_experts, top_k, route_smem + (size_t)wave * num_experts, sel_i,
+                  sel_w);
   if (lane < top_k) {
     topk_ids[(size_t)t * top_k + lane] = sel_i;
-    topk_weights[(size_t)t * top_k + lane] = ssum > 0.0f ? sel_p / ssum : 1.0f / (float)top_k;
+    topk_weights[(size_t)t * top_k + lane] = sel_w;
   }
 }
 

@@ -146,7 +146,10 @@ class MoeBuffers:
 
     def __del__(self):
         if getattr(self, "_h", None) and self._owner:
-            _ffi.lib().xabe_moe_buffers_free(self._h)
+            try:
+                _ffi.lib().xabe_moe_buffers_free(self._h)
+            except Exception:  # interpreter shutdown
+                pass
             self._h = None
 
     def scope(self) -> BufferScope:
@@ -198,7 +201,10 @@ class MoeKernels:
 
     def __del__(self):
         if getattr(self, "_h", None):
-            _ffi.lib().xabe_moe_kernels_free(self._h)
+            try:
+                _ffi.lib().xabe_moe_kernels_free(self._h)
+            except Exception:  # interpreter shutdown
+                pass
             self._h = None
 
     def geometry(self) -> MoeGeometry:

@@ -214,3 +214,43 @@ def test_block_error_paths(oracle, X):
         blk.forward(layer.dev, x[:3], 3, torch.zeros_like(x), torch.zeros_like(x))
     with pytest.raises(X.moe.BufferLength, match="l_out"):
         blk.forward(layer.dev, x, 3, torch.zeros_like(x), torch.zeros_like(x)[:2])
+
+
+@pytest.mark.parametrize("max_tokens,tokens", [(1, 1), (2, 2), (3, 3), (4, 4), (4, 1)])
+def test_fused_shared_is_bit_identical_to_separate_launches(oracle, X, max_tokens, tokens):
+    # crates/xabe-engine/tests/moe_fused_shared_differential.rs:1-20: widths 1..4, full and one live token
+    import torch
+
+    g = X.MoeGeometry.qwen3_6(32, max_tokens)
+    layer = make_layer(oracle, g, seed=720)
+    d = layer.dev
+    x = activations(41, max_tokens, 2048, tokens)
+    rng = np.random.default_rng(max_tokens * 10 + tokens)
+    logits = torch.from_numpy(rng.uniform(-8, 8, (max_tokens, 256)).astype(np.float32)).cuda()
+    outs = []
+    for fused in (True, False):
+        k = X.MoeKernels(g)
+        b = k.buffers()
+        k.set_valid_tokens(b, tokens)
+        k.route_and_dispatch(b, logits)
+        sh = torch.zeros(max_tokens, 2048, device="cuda")
+        if fused:
+            assert k.grouped_forward_partial_with_shared(b, d.gate_exps, d.up_exps, d.down_exps, d.shared_gate,
+                                                         d.shared_up, d.shared_down, x, sh)
+        else:
+            k.grouped_forward_partial(b, d.gate_exps, d.up_exps, d.down_exps, x)
+            k.shared_expert(b, d.shared_gate, d.shared_up, d.shared_down, x, sh)
+        torch.cuda.synchronize()
+        outs.append((b.partial().cpu().numpy()[: tokens * 8 * 2048].copy(), sh.cpu().numpy().copy(),
+                     b.shared_inter().cpu().numpy()[: tokens * 512].copy()))
+    for a, c in zip(outs[0], outs[1]):
+        assert np.array_equal(a.view(np.uint32), c.view(np.uint32))
+    # not covered above the decode width: nothing is launched, the caller takes the separate paths
+    g8 = X.MoeGeometry.qwen3_6(32, 8)
+    k8 = X.MoeKernels(g8)
+    b8 = k8.buffers()
+    x8 = activations(42, 8, 2048)
+    sh8 = torch.zeros(8, 2048, device="cuda")
+    assert not k8.grouped_forward_partial_with_shared(b8, d.gate_exps, d.up_exps, d.down_exps, d.shared_gate, d.shared_up,
+                                                      d.shared_down, x8, sh8)
+    assert torch.all(sh8 == 0)

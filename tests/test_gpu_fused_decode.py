@@ -1,0 +1,95 @@
+"""The decode-width block (max_tokens <= 4) regrouped into three launches against the same block with one
+launch per step: every observable tensor bit for bit, over repeated calls, with fewer live tokens than
+the buffer holds, with and without a logit bias, and for each format pairing.  The per-step launches are
+the ones the oracle comparisons of test_gpu_decode.py cover; test_block_matches_oracle runs the regrouped
+block against the oracle directly."""
+import numpy as np
+import pytest
+
+from util import activations, make_layer, run_block
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def X():
+    import llmxabe_amd as X
+    return X
+
+
+def _observe(blk, g, ffn, lout, tokens):
+    t, k = tokens, g.experts_per_token
+    b = blk.buffers()
+    return dict(
+        ffn=ffn[:t].cpu().numpy(), l_out=lout[:t].cpu().numpy(),
+        normed=blk.normed().view(g.max_tokens, g.hidden)[:t].cpu().numpy(),
+        logits=blk.router_logits().view(g.max_tokens, g.num_experts)[:t].cpu().numpy(),
+        routed=blk.routed().view(g.max_tokens, g.hidden)[:t].cpu().numpy(),
+        shexp=blk.shared_ungated().view(g.max_tokens, g.hidden)[:t].cpu().numpy(),
+        gate=blk.shared_gate().view(-1)[:t].cpu().numpy(),
+        ids=b.topk_ids().view(g.max_tokens, k)[:t].cpu().numpy(),
+        weights=b.topk_weights().view(g.max_tokens, k)[:t].cpu().numpy())
+
+
+def _same_bits(a, b, what):
+    for key in a:
+        x, y = a[key], b[key]
+        if x.dtype == np.float32:
+            x, y = x.view(np.uint32), y.view(np.uint32)
+        assert np.array_equal(x, y), f"{what}: {key} differs"
+
+
+def _compare(X, oracle, g, tokens_seq, seed, router_q8=True, bias=False, expert_quant=None, shared_quant=None):
+    import torch
+
+    layer = make_layer(oracle, g, seed=seed, router_q8=router_q8, expert_quant=expert_quant, shared_quant=shared_quant)
+    one, many = X.MoeBlock(g), X.MoeBlock(g)
+    many.set_fused_decode(False)
+    lb = X.synth_normal_f32(seed + 77, g.num_experts, 1.0) if bias else None
+    for i, tokens in enumerate(tokens_seq):
+        x = activations(seed + 10 + i, g.max_tokens, g.hidden, tokens)
+        f1, l1 = run_block(one, layer, x, tokens, logit_bias=lb)
+        f2, l2 = run_block(many, layer, x, tokens, logit_bias=lb)
+        _same_bits(_observe(one, g, f1, l1, tokens), _observe(many, g, f2, l2, tokens), f"call {i} tokens {tokens}")
+
+
+@pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (2, (2, 1, 2)), (3, (3, 1, 2, 3)), (4, (4, 3, 0, 4, 1))])
+@pytest.mark.parametrize("router_q8", [True, False])
+def test_small_geometry(oracle, X, max_tokens, tokens_seq, router_q8):
+    g = X.MoeGeometry(8, 2, 512, 256, 32, max_tokens)
+    _compare(X, oracle, g, tokens_seq, seed=4100 + max_tokens, router_q8=router_q8, bias=router_q8)
+
+
+@pytest.mark.parametrize("eq,sq", [("Q6K", "Q6K"), ("Q8_0", "Q8_0"), ("Q8_0", "Q6K")])
+def test_small_geometry_format_pairings(oracle, X, eq, sq):
+    g = X.MoeGeometry(16, 4, 512, 256, 32, 3)
+    _compare(X, oracle, g, (3, 2), seed=4200, expert_quant=getattr(X.ExpertQuant, eq), shared_quant=getattr(X.ExpertQuant, sq))
+
+
+@pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (3, (3, 3, 2)), (4, (4, 1, 4))])
+def test_model_geometry(oracle, X, max_tokens, tokens_seq):
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(max_tokens), max_tokens)
+    _compare(X, oracle, g, tokens_seq, seed=4300 + max_tokens, bias=(max_tokens == 3))
+
+
+def test_model_geometry_f32_router(oracle, X):
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(3), 3)
+    _compare(X, oracle, g, (3, 2), seed=4400, router_q8=False)
+
+
+def test_many_replays_keep_the_bits(oracle, X):
+    # 200 back-to-back passes on one stream, no host work between
+    import torch
+
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(3), 3)
+    layer = make_layer(oracle, g, seed=4500)
+    blk = X.MoeBlock(g)
+    x = activations(4511, 3, 2048)
+    ffn, lout = torch.zeros_like(x), torch.zeros_like(x)
+    blk.forward(layer.dev, x, 3, ffn, lout)
+    torch.cuda.synchronize()
+    first = lout.clone()
+    for _ in range(200):
+        blk.forward(layer.dev, x, 3, ffn, lout)
+    torch.cuda.synchronize()
+    assert torch.equal(first.view(torch.int32), lout.view(torch.int32))
