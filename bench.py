@@ -105,51 +105,49 @@ def main() -> int:
     step_bytes = d_active * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES + 16384 + T * 2048 * 4 * 3
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- dominant kernel: routed gate/up GEMV (two of three expert matrices) ----
-    k = X.MoeKernels(g)
-    b = k.buffers()
-    k.set_valid_tokens(b, T)
-    normed = torch.empty_like(x)
-    logits = torch.empty(T, 256, device="cuda")
-    per_layer_bytes = []
+    # ---- the three launches of the block, each timed alone (HIP events on the launch stream, graph replay
+    # over the same rotated layers); the dominant one is launch 1: route + routed gate/up, which streams
+    # two of the three matrices of every (token, k) pair ----
+    pairs = T * 8
+    chunks = (T + 1) // 2  # launch 0 reads the router and the shared gate/up once per chunk of two tokens
+    stage_bytes = [chunks * (ROUTER_BYTES + 2 * (SHARED_BYTES // 3)),
+                   pairs * 2 * EXPERT_MATRIX_BYTES,
+                   pairs * EXPERT_MATRIX_BYTES + T * (SHARED_BYTES // 3)]
+    stage_us = []
     with torch.cuda.stream(stream):
-        def stage0(i):
-            w = layers[i % L]
-            k.grouped_forward_stage(b, w.gate_exps, w.up_exps, w.down_exps, normed, 0)
-
-        # one routing decision per layer, fixed for the measurement
-        w0 = layers[0]
-        X.LayerOpsKernels.rms_norm(x, w0.post_norm, normed, T, 2048, 1e-6)
-        k.router_logits(b, w0.router, w0.router_quant, normed, logits)
-        k.route_and_dispatch(b, logits)
+        one_pass(0)  # leaves layer 0's logits, normalised rows and shared activations for stages 1 and 2
         stream.synchronize()
-        pairs = T * 8
-        kern_bytes = pairs * 2 * EXPERT_MATRIX_BYTES  # the flat kernel streams gate+up once per (token, k) pair
-        kgraph = torch.cuda.CUDAGraph()
-        for i in range(L):
-            stage0(i)
-        stream.synchronize()
-        with torch.cuda.graph(kgraph, stream=stream):
+        for st in range(3):
+            def run_stage(i, st=st):
+                blk.forward_stage(layers[i % L], x, ffn_out, l_out, st)
             for i in range(L):
-                stage0(i)
-        kgraph.replay()
-        stream.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        kreps = 20
-        e0.record(stream)
-        for _ in range(kreps):
+                run_stage(i)
+            stream.synchronize()
+            kgraph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(kgraph, stream=stream):
+                for i in range(L):
+                    run_stage(i)
             kgraph.replay()
-        e1.record(stream)
-        e1.synchronize()
-        kern_us = e0.elapsed_time(e1) * 1e3 / (kreps * L)
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            kreps = 20
+            e0.record(stream)
+            for _ in range(kreps):
+                kgraph.replay()
+            e1.record(stream)
+            e1.synchronize()
+            stage_us.append(e0.elapsed_time(e1) * 1e3 / (kreps * L))
+    kern_bytes, kern_us = stage_bytes[1], stage_us[1]
     achieved = kern_bytes / (kern_us * 1e-6) / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get("k_expert_flat_gateup_b3_bytes_per_launch")
+            traffic = json.load(open(tpath)).get("k_decode_up_b3_bytes_per_launch")
         except Exception:
             traffic = None
+    stage_names = ["k_decode_logits (router logits + shared gate/up)", "k_decode_up (route + routed gate/up)",
+                   "k_decode_down (routed + shared down, combine)"]
 
     out = {
         "metric": "MoE-block tokens/s at 1 GPU; decode HBM GB/s %peak; prefill MFMA util %",
@@ -171,9 +169,11 @@ def main() -> int:
                    "block_gbps": step_gbps, "block_frac_of_hbm_peak": step_gbps / HBM_PEAK_GBPS,
                    "roofline_tokens_per_s": T / (step_bytes / (HBM_PEAK_GBPS * 1e9)),
                    "frac_of_roofline": tokens_per_s / (T / (step_bytes / (HBM_PEAK_GBPS * 1e9)))},
-        "roofline": {"kernel": "k_expert_flat<Q6_K,K=2048,gate+up>", "bound": "hbm", "achieved": achieved,
+        "roofline": {"kernel": "k_decode_up<Q6_K,hidden 2048> (route + routed gate/up)", "bound": "hbm", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": kern_bytes, "launch_us": kern_us},
+        "launches": [{"kernel": n, "launch_us": u, "algorithmic_bytes": int(bts), "gbps": bts / (u * 1e-6) / 1e9}
+                     for n, u, bts in zip(stage_names, stage_us, stage_bytes)],
     }
 
     if not args.no_cpu:

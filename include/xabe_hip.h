@@ -231,6 +231,13 @@ int xabe_moe_block_set_exact_decode_regime(xabe_moe_block* blk, int on); /* B:10
  * combine) that compute the same values bit for bit.  `on` = 0 keeps one launch per step as the reference
  * has them (B:1091-1329); the switch exists for tests and measurement. */
 int xabe_moe_block_set_fused_decode(xabe_moe_block* blk, int on);
+/* Measurement hook, no counterpart in the reference: ONE of the three decode launches (0: logits + shared
+ * gate/up, 1: route + gate/up, 2: down + combine) with the arguments of xabe_moe_block_forward, so that a
+ * launch can be timed and profiled alone.  Stage n reads what stages < n of an earlier call left in the
+ * block's buffers; the live-token count is the one last published. */
+int xabe_moe_block_forward_stage(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w,
+                                 const float* residual, size_t residual_len, const float* logit_bias, float* ffn_out,
+                                 size_t ffn_out_len, float* l_out, size_t l_out_len, int stage);
 int xabe_moe_block_tensor_cores_enabled(const xabe_moe_block* blk);      /* B:1008-1010 */
 /* Read-back accessors (B:1023-1060): device pointer + element count. */
 const float* xabe_moe_block_normed(const xabe_moe_block* blk, size_t* len);

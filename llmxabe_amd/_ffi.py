@@ -94,6 +94,7 @@ _SIGNATURES = {
     "xabe_moe_block_disable_tensor_cores": (C.c_int, [vp]),
     "xabe_moe_block_set_exact_decode_regime": (C.c_int, [vp, C.c_int]),
     "xabe_moe_block_set_fused_decode": (C.c_int, [vp, C.c_int]),
+    "xabe_moe_block_forward_stage": (C.c_int, [vp, vp, vp, vp, sz, vp, vp, sz, vp, sz, C.c_int]),
     "xabe_moe_block_tensor_cores_enabled": (C.c_int, [vp]),
     "xabe_moe_block_normed": (vp, [vp, C.POINTER(sz)]),
     "xabe_moe_block_router_logits": (vp, [vp, C.POINTER(sz)]),

@@ -71,6 +71,13 @@ class MoeBlock:
                                                 _ptr(logit_bias), _ptr(ffn_out), ffn_out.numel(), _ptr(l_out),
                                                 l_out.numel()))
 
+    def forward_stage(self, w: MoeLayerWeights, residual, ffn_out, l_out, stage: int, logit_bias=None):
+        """One of the three decode launches alone (measurement hook; see the header)."""
+        cw = w._c()
+        check(_ffi.lib().xabe_moe_block_forward_stage(self._h, _stream(), C.byref(cw), _ptr(residual), residual.numel(),
+                                                      _ptr(logit_bias), _ptr(ffn_out), ffn_out.numel(), _ptr(l_out),
+                                                      l_out.numel(), stage))
+
     def _view(self, name: str) -> torch.Tensor:
         n = C.c_size_t(0)
         p = getattr(_ffi.lib(), "xabe_moe_block_" + name)(self._h, C.byref(n))

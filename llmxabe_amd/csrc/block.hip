@@ -68,6 +68,20 @@ static int blk_check_len(const char* what, size_t expected, size_t found) {
   return XABE_OK;
 }
 
+int xabe_moe_block_forward_stage(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
+                                 size_t residual_len, const float* logit_bias, float* ffn_out, size_t ffn_out_len,
+                                 float* l_out, size_t l_out_len, int stage) {
+  if (!blk || !w || !residual || !ffn_out || !l_out) return set_error(XABE_ERR_INVALID_ARGUMENT, "forward_stage: null pointer");
+  if (stage < 0 || stage > 2) return set_error(XABE_ERR_INVALID_ARGUMENT, "forward_stage: stage %d is not 0, 1 or 2", stage);
+  XABE_TRY(blk_check_len("residual", blk->n_act, residual_len));
+  XABE_TRY(blk_check_len("ffn_out", blk->n_act, ffn_out_len));
+  XABE_TRY(blk_check_len("l_out", blk->n_act, l_out_len));
+  if (!decode_block_supported(blk->moe, blk->buffers, w))
+    return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "forward_stage: this geometry does not take the three-launch decode path");
+  return launch_decode_block(blk->moe, as_stream(stream), blk->buffers, w, residual, logit_bias, blk->eps, blk->normed,
+                             blk->logits, blk->shexp, blk->gate, blk->routed, ffn_out, l_out, 1u << stage);
+}
+
 int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
                            size_t residual_len, size_t tokens, const float* logit_bias, float* ffn_out,
                            size_t ffn_out_len, float* l_out, size_t l_out_len) {

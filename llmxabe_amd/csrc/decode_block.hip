@@ -107,7 +107,8 @@ template <int QUANT, int RPS, int TC, int NM>
 __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, int K,
                                             int n_rows, int row0, const float* const (&xrow)[TC],
                                             const float* __restrict__ norm_w, float eps, float* const (&out)[TC],
-                                            const float* __restrict__ bias) {
+                                            const float* __restrict__ bias, const int* __restrict__ valid_tokens,
+                                            int token0) {
   using F = Fmt<QUANT>;
   using Raw = typename F::Raw;
   constexpr int G = 64 / RPS;
@@ -154,13 +155,16 @@ __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, cons
 #pragma unroll
     for (int t = 0; t < TC; ++t) tot[m][t] = group_sum<G>(tot[m][t]);
   }
+  // the live-token count was requested first and is only needed here: rows past it were computed from
+  // whatever the buffer held (in bounds, sized for max_tokens) and are dropped
+  const int valid = *valid_tokens;
   const int row = row0 + g.lane / G;
   if ((g.lane % G) == 0 && row < n_rows) {
 #pragma unroll
     for (int t = 0; t < TC; ++t) {
       float v = NM == 2 ? silu_f(tot[0][t]) * tot[NM - 1][t] : 1.0f * tot[0][t];
       if (NM == 1 && bias) v += bias[row];
-      out[t][row] = v;
+      if (token0 + t < valid) out[t][row] = v;
     }
   }
 }
@@ -172,7 +176,6 @@ __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, cons
 template <int SQ, int RF, int RPS>
 __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
   __shared__ float s_red[4];
-  const int valid = *a.valid_tokens;
   const int chunks = (a.max_tokens + 1) / 2;
   const int n_r = chunks * a.tiles_r;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -183,26 +186,25 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
     if (!router) item -= n_r;
     const int tiles = router ? a.tiles_r : a.tiles_s;
     const int c = item / tiles, tile = item % tiles, t0 = 2 * c;
-    if (t0 >= valid) return;
     const int row0 = (tile * kWavesPerWg + wave) * RPS;
     const float* x0 = a.residual + (size_t)t0 * a.H;
-    if (t0 + 1 < valid) {
+    if (t0 + 1 < a.max_tokens) {
       const float* const xr[2] = {x0, x0 + a.H};
       if (router) {
         float* const o[2] = {a.logits + (size_t)t0 * a.E, a.logits + (size_t)(t0 + 1) * a.E};
-        step_normed<RF, RPS, 2, 1>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias);
+        step_normed<RF, RPS, 2, 1>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0);
       } else {
         float* const o[2] = {a.shared_inter + (size_t)t0 * a.I, a.shared_inter + (size_t)(t0 + 1) * a.I};
-        step_normed<SQ, RPS, 2, 2>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr);
+        step_normed<SQ, RPS, 2, 2>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0);
       }
     } else {
       const float* const xr[1] = {x0};
       if (router) {
         float* const o[1] = {a.logits + (size_t)t0 * a.E};
-        step_normed<RF, RPS, 1, 1>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias);
+        step_normed<RF, RPS, 1, 1>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0);
       } else {
         float* const o[1] = {a.shared_inter + (size_t)t0 * a.I};
-        step_normed<SQ, RPS, 1, 2>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr);
+        step_normed<SQ, RPS, 1, 2>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0);
       }
     }
     XABE_TRACE(0, 3);
@@ -211,7 +213,7 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
   // the normalised row (callers read it back) and g = sigmoid(shared_gate_inp . normed): the order of
   // operations of the stand-alone RMSNorm and gate kernels
   const int t = blockIdx.x;
-  if (t >= valid) return;
+  const int valid = *a.valid_tokens;
   const float* xr = a.residual + (size_t)t * a.H;
   // hidden <= 2048: eight columns per thread, every load issued before the first use
   float xv[8], nv[8], gv[8];
@@ -224,6 +226,7 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
     gv[i] = in ? a.shared_gate_inp[j] : 0.0f;
   }
   const float inv = row_inv_rms(xr, a.H, a.eps);
+  if (t >= valid) return;
   float s = 0.0f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -254,17 +257,30 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   __shared__ int s_expert;
   const int p = blockIdx.x / a.tiles_g, tile = blockIdx.x % a.tiles_g;
   const int t = p / a.top_k, k = p % a.top_k;
-  if (t >= *a.valid_tokens) return;
+  // everything read before the live-token count is known is sized for max_tokens rows
+  const int valid = *a.valid_tokens;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const LaneGeom g = lane_geom<RQ>();
   const int koff = lane_koff<RQ, RPS>(g, 0);
   XABE_TRACE(1, 0);
-  // route the token on one wavefront (a different one in neighbouring workgroups, which share a CU)
-  if (wave == (int)((blockIdx.x >> 8) & 3)) {
+  // one wavefront routes the token (a different one in neighbouring workgroups, which share a CU); its
+  // logits and every wavefront's copy of the normalised row are requested together
+  const bool routes = wave == (int)((blockIdx.x >> 8) & 3);
+  const bool few = a.E <= 256;
+  float lg[kRouteMaxPerLane];
+  if (routes) {
+    if (few) route_load<4>(a.logits + (size_t)t * a.E, a.E, nullptr, nullptr, *reinterpret_cast<float(*)[4]>(lg));
+    else route_load<kRouteMaxPerLane>(a.logits + (size_t)t * a.E, a.E, nullptr, nullptr, lg);
+  }
+  float x[1][32], xs[1][4];
+  lane_x_load<RQ>(a.normed + (size_t)t * a.H, koff, g, x[0]);
+  if (t >= valid) return;
+  if (routes) {
     int sel_i;
     float sel_w;
     XABE_ROUTE_TRACE(0);
-    route_one_token(a.logits + (size_t)t * a.E, a.E, a.top_k, s_route, sel_i, sel_w);
+    if (few) route_compute<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, a.top_k, s_route, sel_i, sel_w);
+    else route_compute<kRouteMaxPerLane>(lg, a.E, a.top_k, s_route, sel_i, sel_w);
     XABE_ROUTE_TRACE(5);
     if (g.lane == k) s_expert = sel_i;
     if (k == 0 && tile == 0 && g.lane < a.top_k) {
@@ -272,10 +288,9 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
       a.topk_weights[(size_t)t * a.top_k + g.lane] = sel_w;
     }
   }
+  lane_x_offsets<RQ>(x[0], xs[0]);
   __syncthreads();
   XABE_TRACE(1, 1);
-  float x[1][32], xs[1][4];
-  lane_x_load<RQ>(a.normed + (size_t)t * a.H, koff, g, x[0]);
   const int e = s_expert;
   const size_t row_bytes = (size_t)(a.H / F::kBlockElems) * F::kBlockBytes;
   const uint8_t* wg = a.gate + (size_t)e * a.expert_bytes;
@@ -284,12 +299,10 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   Raw r[DEPTH][2];
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
-    const int row0 = wave_row0 + d * RPS;
-    const bool live = row0 < a.I;
-    load_raw<RQ>(wg + (size_t)row0 * row_bytes, live, g, r[d][0]);
-    load_raw<RQ>(wu + (size_t)row0 * row_bytes, live, g, r[d][1]);
+    const int row0 = wave_row0 + d * RPS;  // the tiles divide the rows exactly (checked by the host)
+    load_raw<RQ>(wg + (size_t)row0 * row_bytes, true, g, r[d][0]);
+    load_raw<RQ>(wu + (size_t)row0 * row_bytes, true, g, r[d][1]);
   }
-  lane_x_offsets<RQ>(x[0], xs[0]);
   float* out = a.inter + (size_t)p * a.I;
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
@@ -354,7 +367,9 @@ __global__ void __launch_bounds__(256) k_decode_down(DecodeArgs a) {
 #pragma unroll
   for (int k = 0; k < kMaxTopK; ++k) {
     const int e = min(max(__builtin_amdgcn_readlane(my_e, k), 0), a.E - 1);
-    load_raw<RQ>(a.down + (size_t)e * a.expert_bytes + (size_t)row0 * rb_r, k < a.top_k, gr, rr[k]);
+    // k >= top_k reads expert 0's rows and never uses them: an unconditional load keeps all of round two
+    // in one basic block, so every load is issued before the first wait
+    load_raw<RQ>(a.down + (size_t)e * a.expert_bytes + (size_t)row0 * rb_r, true, gr, rr[k]);
   }
   // the activation rows arrived before the weights (loads return in order); publish them to LDS
 #pragma unroll
@@ -403,13 +418,14 @@ struct Launch {
   hipStream_t s;
   unsigned grid_a, grid_b, grid_c;
   size_t route_lds;
+  unsigned launches;  // bit i: issue launch i (A, B, C); all three outside measurements
 };
 
 template <int RQ, int SQ, int RF, int RPSH, int DEPTH, int RPSI>
 static void launch_all(const Launch& l) {
-  hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);
-  hipLaunchKernelGGL((k_decode_up<RQ, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
-  hipLaunchKernelGGL((k_decode_down<RQ, SQ, RPSI>), dim3(l.grid_c), dim3(256), 0, l.s, l.a);
+  if (l.launches & 1u) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);
+  if (l.launches & 2u) hipLaunchKernelGGL((k_decode_up<RQ, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
+  if (l.launches & 4u) hipLaunchKernelGGL((k_decode_down<RQ, SQ, RPSI>), dim3(l.grid_c), dim3(256), 0, l.s, l.a);
 }
 
 template <int RQ, int SQ, int RF>
@@ -447,7 +463,7 @@ bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b
 
 int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, const xabe_moe_layer_weights* w,
                         const float* residual, const float* logit_bias, float eps, float* normed, float* logits,
-                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out) {
+                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches) {
   const xabe_moe_geometry& g = k->g;
   DecodeArgs a;
   memset(&a, 0, sizeof(a));
@@ -488,11 +504,11 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
   const int depth = a.H == 2048 ? 4 : 1;  // steps per wavefront of the gate/up launch (launch_shape)
   a.tiles_g = (a.I + kWavesPerWg * depth * rps_h - 1) / (kWavesPerWg * depth * rps_h);
   a.tiles_d = (a.H + kWavesPerWg * rps_i - 1) / (kWavesPerWg * rps_i);
-  if (a.E % rps_h != 0 || a.I % rps_h != 0)
+  if (a.E % rps_h != 0 || a.I % (kWavesPerWg * depth * rps_h) != 0 || a.H % (kWavesPerWg * rps_i) != 0)
     return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "decode block: %d experts / %d intermediate rows do not fill whole steps of %d rows",
                      a.E, a.I, rps_h);
   const int chunks = (a.max_tokens + 1) / 2;
-  Launch l{a, s, 0, 0, 0, g.num_experts * sizeof(float)};
+  Launch l{a, s, 0, 0, 0, g.num_experts * sizeof(float), launches};
   l.grid_a = (unsigned)(chunks * (a.tiles_r + a.tiles_s) + a.max_tokens);
   l.grid_b = (unsigned)(a.max_tokens * a.top_k * a.tiles_g);
   l.grid_c = (unsigned)(a.max_tokens * a.tiles_d);

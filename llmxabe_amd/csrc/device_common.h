@@ -146,13 +146,14 @@ __device__ __forceinline__ void load8_funnel(const uint8_t* base4, uint32_t off,
   hi = __builtin_amdgcn_alignbit(d2, d1, sh);
 }
 // Same, but never touches the third dword unless the field really spills into it
-// (the last field of the last block of a tensor must not be over-read).
+// (the last field of the last block of a tensor must not be over-read).  Branch-free: an aligned field
+// reads its second dword twice instead; a branch here would end the basic block and make the compiler
+// wait for each block's loads before issuing the next block's.
 __device__ __forceinline__ void load8_funnel_tail(const uint8_t* base4, uint32_t off, uint32_t& lo, uint32_t& hi) {
   const uint32_t a = off & ~3u, sh = (off & 2u) << 3;
   const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + a);
   const uint32_t d0 = p[0], d1 = p[1];
-  uint32_t d2 = 0;
-  if (sh) d2 = p[2];
+  const uint32_t d2 = p[sh ? 2 : 1];
   lo = __builtin_amdgcn_alignbit(d1, d0, sh);
   hi = __builtin_amdgcn_alignbit(d2, d1, sh);
 }
@@ -260,9 +261,9 @@ __device__ __forceinline__ void q8_load(const uint8_t* chunk4, uint32_t lane_off
 #pragma unroll
   for (int i = 0; i < 8; ++i) e[i] = p[i];
   // The ninth piece is the block's last two codes only: a dword there would read two
-  // bytes past the last block of a tensor.
-  e[8] = 0;
-  if (sh) e[8] = load_u16(chunk4, lane_off + 32);
+  // bytes past the last block of a tensor.  Unused (and aimed at the block's first bytes, no branch) when
+  // the codes are dword-aligned.
+  e[8] = load_u16(chunk4, lane_off + (sh ? 32u : 0u));
 #pragma unroll
   for (int i = 0; i < 8; ++i) r.q[i] = __builtin_amdgcn_alignbit(e[i + 1], e[i], sh);
   r.dh = load_u16(chunk4, lane_off);

@@ -58,7 +58,7 @@ int pick_tile_rows(const xabe_moe_kernels* k, size_t live_units, int n_rows, int
 bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, const xabe_moe_layer_weights* w);
 int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, const xabe_moe_layer_weights* w,
                         const float* residual, const float* logit_bias, float eps, float* normed, float* logits,
-                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out);
+                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches = 7u);
 
 // matrix-core regime (mfma.hip)
 bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int gate_q, int up_q, int down_q, bool routed);
