@@ -37,6 +37,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=16, help="independent weight sets rotated through")
     ap.add_argument("--tokens", type=int, default=3)
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a hipGraph")
+    ap.add_argument("--calibration-copies", type=int, default=0,
+                    help="before the timed region, copy a 256 MiB device buffer this many times: a kernel of known "
+                         "traffic against which hardware byte counters of the same run are scaled")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -62,6 +65,12 @@ def main() -> int:
     blk.publish_tokens(T)
     ffn_out = torch.zeros_like(x)
     l_out = torch.zeros_like(x)
+    if args.calibration_copies:
+        src = torch.zeros(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.calibration_copies):
+            dst.copy_(src)
+        del src, dst
     torch.cuda.synchronize()   # the generators ran on the default stream; the timed work uses its own
 
     def one_pass(i):
