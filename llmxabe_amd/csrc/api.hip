@@ -121,6 +121,33 @@ static void launch_shape(Shape shape, Mode mode, dim3 grid, hipStream_t s, const
   }
 }
 
+// Dispatch-table regime, rows of one step: the weights-resident kernel where its tile divides the rows.
+template <int QUANT, int NM>
+static bool launch_block_resident(Shape shape, const ExpertArgs& a, size_t units, hipStream_t s) {
+  if (shape == kKs2 || shape == kStream || a.K * rows_per_step(shape) != 2048) return false;
+  const int rps = rows_per_step(shape);
+  // steps per wavefront: as many as keep the raw bytes of a tile within ~36 registers per lane
+  const int want = NM == 2 ? 2 : 4;
+  const int depth = a.n_rows % (kWavesPerWg * want * rps) == 0 ? want : a.n_rows % (kWavesPerWg * 2 * rps) == 0 ? 2 : 0;
+  if (!depth) return false;
+  const unsigned tiles = (unsigned)(a.n_rows / (kWavesPerWg * depth * rps));
+  if (tiles > 65535u || units > 65535u) return false;
+  dim3 grid(tiles, (unsigned)units);
+#define XABE_RESIDENT(RPS)                                                                                         \
+  do {                                                                                                             \
+    if (depth == 4) hipLaunchKernelGGL((k_expert_block_resident<QUANT, RPS, NM, 4>), grid, dim3(256), 0, s, a);    \
+    else hipLaunchKernelGGL((k_expert_block_resident<QUANT, RPS, NM, 2>), grid, dim3(256), 0, s, a);               \
+  } while (0)
+  switch (shape) {
+    case kRps8: XABE_RESIDENT(8); break;
+    case kRps4: XABE_RESIDENT(4); break;
+    case kRps2: XABE_RESIDENT(2); break;
+    default: XABE_RESIDENT(1); break;
+  }
+#undef XABE_RESIDENT
+  return true;
+}
+
 int pick_tile_rows(const xabe_moe_kernels* k, size_t live_units, int n_rows, int rps) {
   // aim for ~12 wavefronts per CU across the launch
   const size_t items = std::max<size_t>(1, live_units) * (size_t)n_rows / rps;
@@ -137,6 +164,15 @@ static int launch_expert(const xabe_moe_kernels* k, Mode mode, int quant, int nm
                          size_t live_units, hipStream_t s) {
   const Shape shape = shape_for((size_t)a.K);
   const int rps = rows_per_step(shape);
+  if (mode == kBlock && !k->force_community) {
+    bool done = false;
+    if (quant == XABE_QUANT_Q6K) done = nm == 2 ? launch_block_resident<kQ6K, 2>(shape, a, units, s) : launch_block_resident<kQ6K, 1>(shape, a, units, s);
+    else if (quant == XABE_QUANT_Q8_0) done = nm == 2 ? launch_block_resident<kQ8_0, 2>(shape, a, units, s) : launch_block_resident<kQ8_0, 1>(shape, a, units, s);
+    if (done) {
+      XABE_HIP_TRY(hipGetLastError());
+      return XABE_OK;
+    }
+  }
   a.tile_rows = pick_tile_rows(k, live_units, a.n_rows, rps);
   const unsigned tiles = (unsigned)((a.n_rows + a.tile_rows - 1) / a.tile_rows);
   if (tiles > 65535) return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "row-tile count %u exceeds the grid.y limit", tiles);

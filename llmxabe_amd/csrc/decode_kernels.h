@@ -387,6 +387,97 @@ __global__ void __launch_bounds__(256) k_expert_block(ExpertArgs a) {
   }
 }
 
+// The same dispatch-table work unit with the weights resident: a workgroup's tile is exactly what its four
+// wavefronts can hold in registers (DEPTH steps each), every weight byte is requested before the first wait,
+// and the block's token chunks then run against those registers -- the weights are read once per block
+// instead of once per chunk, and a wavefront's loads are all in flight together instead of one step at a
+// time.  Rows of at most 2048 elements (one step); n_rows must be a multiple of 4 * DEPTH * RPS.
+// The per-row arithmetic is matvec_rows', so the outputs are bit-identical to k_expert_block's.
+template <int N>
+struct TcC {
+  static constexpr int value = N;
+};
+
+template <int QUANT, int RPS, int NM, int DEPTH>
+__global__ void __launch_bounds__(256) k_expert_block_resident(ExpertArgs a) {
+  using F = Fmt<QUANT>;
+  using Raw = typename F::Raw;
+  constexpr int G = 64 / RPS;
+  const int b = blockIdx.y;
+  const int* slots = a.sorted_token_ids + (size_t)b * a.block_size;
+  const int e = a.expert_ids[b];
+  int f0 = slots[0], f1 = a.block_size > 1 ? slots[1] : 0x7fffffff;
+  const int valid = *a.valid_tokens;
+  if (e < 0) return;
+  const int sentinel = valid * a.top_k;
+  if (f0 >= sentinel) return;
+  const LaneGeom g = lane_geom<QUANT>();
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int koff = lane_koff<QUANT, RPS>(g, 0);
+  const size_t row_bytes = (size_t)(a.K / F::kBlockElems) * F::kBlockBytes;
+  const uint8_t* w0 = a.w0 + (size_t)e * a.expert_bytes;
+  const uint8_t* w1 = NM == 2 ? a.w1 + (size_t)e * a.expert_bytes : nullptr;
+  const int wave_row0 = ((int)blockIdx.x * kWavesPerWg + wave) * DEPTH * RPS;
+  // a chunk's activation rows (the second repeats the first in a one-token chunk: loaded, never used)
+  float x[2][32], xs[2][4];
+  bool two;
+  auto load_chunk = [&](int i) {
+    two = f1 < sentinel;
+    const size_t s0 = (size_t)b * a.block_size + i;
+    load_x<QUANT>(a.x + (NM == 2 ? (size_t)(f0 / a.top_k) : s0) * a.K, koff, true, g, x[0], xs[0]);
+    load_x<QUANT>(a.x + (NM == 2 ? (size_t)((two ? f1 : f0) / a.top_k) : (two ? s0 + 1 : s0)) * a.K, koff, true, g, x[1], xs[1]);
+  };
+  load_chunk(0);  // requested ahead of the weights, so it is there when they arrive
+  Raw r[DEPTH][NM];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) {
+    const size_t off = (size_t)(wave_row0 + d * RPS) * row_bytes;
+    load_raw<QUANT>(w0 + off, true, g, r[d][0]);
+    if constexpr (NM == 2) load_raw<QUANT>(w1 + off, true, g, r[d][NM - 1]);
+  }
+  for (int i = 0;;) {
+    const size_t s0 = (size_t)b * a.block_size + i;
+    auto chunk = [&](auto tc_c) {
+      constexpr int TC = decltype(tc_c)::value;
+      const int f[2] = {f0, f1};
+      const float (&xt)[TC][32] = *reinterpret_cast<const float (*)[TC][32]>(&x);
+      const float (&xst)[TC][4] = *reinterpret_cast<const float (*)[TC][4]>(&xs);
+      float* o[TC];
+      float sc[TC];
+#pragma unroll
+      for (int t = 0; t < TC; ++t) {
+        o[t] = a.out + (NM == 2 ? s0 + t : (size_t)f[t]) * a.n_rows;
+        sc[t] = NM == 2 ? 1.0f : a.topk_weights[f[t]];
+      }
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        float tot[NM][TC];
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+#pragma unroll
+          for (int t = 0; t < TC; ++t) tot[m][t] = 0.0f;
+          accum<QUANT, TC>(r[d][m], g, xt, xst, tot[m]);
+#pragma unroll
+          for (int t = 0; t < TC; ++t) tot[m][t] = group_sum<G>(tot[m][t]);
+        }
+        const int row = wave_row0 + d * RPS + g.lane / G;
+        if ((g.lane % G) == 0) {
+#pragma unroll
+          for (int t = 0; t < TC; ++t) o[t][row] = NM == 2 ? silu_f(tot[0][t]) * tot[NM - 1][t] : sc[t] * tot[0][t];
+        }
+      }
+    };
+    if (two) chunk(TcC<2>{});
+    else chunk(TcC<1>{});
+    i += 2;
+    if (i >= a.block_size) break;
+    f0 = slots[i];
+    f1 = (i + 1 < a.block_size) ? slots[i + 1] : sentinel;
+    if (f0 >= sentinel) break;
+    load_chunk(i);
+  }
+}
+
 // Shared expert / dense MLP: every live token, no indirection, no routing weight
 // (crates/xabe-cuda/src/kernels/moe.rs:3425-3725, :4082-4227).  One work unit per chunk of two tokens.
 template <int QUANT, int KS, int RPS, int NM>

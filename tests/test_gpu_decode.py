@@ -254,3 +254,34 @@ def test_fused_shared_is_bit_identical_to_separate_launches(oracle, X, max_token
     assert not k8.grouped_forward_partial_with_shared(b8, d.gate_exps, d.up_exps, d.down_exps, d.shared_gate, d.shared_up,
                                                       d.shared_down, x8, sh8)
     assert torch.all(sh8 == 0)
+
+
+@pytest.mark.parametrize("geom,max_tokens,tokens", [("model", 8, 8), ("model", 32, 29), ("small", 40, 40), ("small", 5, 5)])
+def test_weights_resident_dispatch_kernel_equals_the_plain_one(oracle, X, geom, max_tokens, tokens):
+    # the dispatch-table regime (5..63 tokens) keeps a tile's weights in registers across the block's token
+    # chunks; force_community selects the plain per-chunk kernel: same bits, both stages
+    import torch
+
+    if geom == "model":
+        g = X.MoeGeometry.qwen3_6(X.moe_block_size(max_tokens), max_tokens)
+    else:
+        g = X.MoeGeometry(8, 2, 512, 256, 32, max_tokens)  # few experts: long runs, several chunks per block
+    layer = make_layer(oracle, g, seed=733)
+    x = activations(44, max_tokens, g.hidden, tokens)
+    r = oracle.Xorshift64Star(0xB22 + tokens)
+    logits = np.stack([r.vec_f32(g.num_experts, -8.0, 8.0) for _ in range(tokens)])
+    outs = []
+    for plain in (False, True):
+        k = X.MoeKernels(g)
+        k.force_community(plain)
+        b = k.buffers()
+        k.set_valid_tokens(b, tokens)
+        lg = torch.zeros(max_tokens, g.num_experts, device="cuda")
+        lg[:tokens] = torch.from_numpy(logits).cuda()
+        k.route_and_dispatch(b, lg)
+        d = layer.dev
+        k.grouped_forward_partial(b, d.gate_exps, d.up_exps, d.down_exps, x)
+        torch.cuda.synchronize()
+        outs.append(b.partial().cpu().numpy().copy())
+    assert outs[0].any()
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
