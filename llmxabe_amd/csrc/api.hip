@@ -382,6 +382,9 @@ static int alloc_buffers(const xabe_moe_kernels* k, void* stream, int scope, boo
   A(&b->expert_ids, b->n_expert_blocks);
   A(&b->bucket_live, b->n_expert_blocks);
   A(&b->expert_counts, routed ? g.num_experts : 0);
+  // the counting-sort form of the dispatch tables, from 8192 selections up
+  b->n_align_chunks = (routed && flat >= 8192 && g.num_experts <= 512) ? (flat + 1023) / 1024 : 0;
+  A(&b->align_hist, b->n_align_chunks * g.num_experts);
   A(&b->num_tokens_post_pad, routed ? 1 : 0);
   A(&b->valid_tokens, 1);
   A(&b->inter, b->n_inter);
@@ -412,7 +415,7 @@ int xabe_moe_shared_only_buffers_new(const xabe_moe_kernels* k, void* stream, in
 void xabe_moe_buffers_free(xabe_moe_buffers* b) {
   if (!b) return;
   void* ptrs[] = {b->topk_ids, b->topk_weights, b->sorted_token_ids, b->expert_ids, b->bucket_live, b->expert_counts,
-                  b->num_tokens_post_pad, b->valid_tokens, b->inter, b->partial, b->shared_inter, b->x_h, b->inter_h,
+                  b->num_tokens_post_pad, b->valid_tokens, b->align_hist, b->inter, b->partial, b->shared_inter, b->x_h, b->inter_h,
                   b->shared_inter_h, b->tile_list};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
@@ -472,6 +475,19 @@ int xabe_moe_build_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_bu
   XABE_TRY(require_routed(b, "build_dispatch"));
   const xabe_moe_geometry& g = k->g;
   hipStream_t s = as_stream(stream);
+  if (b->n_align_chunks) {
+    const unsigned chunks = (unsigned)b->n_align_chunks;
+    hipLaunchKernelGGL(k_align_hist, dim3(chunks), dim3(256), 0, s, b->topk_ids, b->valid_tokens, (int)g.experts_per_token,
+                       (int)g.num_experts, (int)b->n_sorted, (int)b->n_expert_blocks, b->align_hist, b->sorted_token_ids,
+                       b->expert_ids, b->bucket_live);
+    hipLaunchKernelGGL(k_align_offsets, dim3(1), dim3(512), 0, s, b->valid_tokens, (int)g.experts_per_token,
+                       (int)g.num_experts, (int)g.block_size, (int)chunks, (int)b->n_expert_blocks, b->align_hist,
+                       b->expert_counts, b->expert_ids, b->bucket_live, b->num_tokens_post_pad);
+    hipLaunchKernelGGL(k_align_place, dim3(chunks), dim3(256), 0, s, b->topk_ids, b->valid_tokens, (int)g.experts_per_token,
+                       (int)g.num_experts, (int)b->n_sorted, b->align_hist, b->sorted_token_ids);
+    XABE_HIP_TRY(hipGetLastError());
+    return XABE_OK;
+  }
   hipLaunchKernelGGL(k_align_count, dim3((unsigned)g.num_experts), dim3(256), 0, s, b->topk_ids, b->valid_tokens,
                      (int)g.experts_per_token, (int)b->n_sorted, (int)b->n_expert_blocks, b->sorted_token_ids,
                      b->expert_ids, b->bucket_live, b->expert_counts);

@@ -90,6 +90,8 @@ struct xabe_moe_buffers {
   int32_t* expert_ids;
   int32_t* bucket_live;
   int32_t* expert_counts;
+  int32_t* align_hist;      // [chunks of 1024 selections][num_experts], prefill widths only
+  size_t n_align_chunks;
   int32_t* num_tokens_post_pad;
   int32_t* valid_tokens;
   int32_t valid_published;

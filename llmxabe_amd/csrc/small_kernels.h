@@ -142,6 +142,144 @@ __global__ void __launch_bounds__(256) k_align_scatter(const int* __restrict__ t
 }
 
 // ---------------------------------------------------------------------------------
+// The same dispatch tables for prefill widths, as a stable counting sort in three launches whose work is
+// proportional to the number of selections (the two-launch form above has every expert's workgroup scan all
+// of them).  A chunk is 1024 consecutive flat ids, 256 per wavefront.
+//   hist:    per-chunk, per-expert counts; whole-capacity sentinel / -1 / 0 fill.
+//   offsets: one workgroup: per-expert totals, the exclusive prefix of the padded totals, every chunk's
+//            first slot per expert, the block tables.
+//   place:   per chunk: each wavefront ranks its ids among equals in index order and writes them.
+// No result depends on the order in which atomics land, so the tables are the CPU reference's.
+// ---------------------------------------------------------------------------------
+constexpr int kAlignChunk = 1024;
+constexpr int kAlignMaxExperts = 512;
+
+__global__ void __launch_bounds__(256) k_align_hist(const int* __restrict__ topk_ids, const int* __restrict__ valid_tokens,
+                                                     int top_k, int num_experts, int sorted_capacity, int expert_capacity,
+                                                     int* __restrict__ chunk_hist, int* __restrict__ sorted_token_ids,
+                                                     int* __restrict__ expert_ids, int* __restrict__ bucket_live) {
+  __shared__ int hist[kAlignMaxExperts];
+  const int numel = *valid_tokens * top_k;
+  for (int e = threadIdx.x; e < num_experts; e += 256) hist[e] = 0;
+  __syncthreads();
+  const int i0 = blockIdx.x * kAlignChunk;
+  for (int j = threadIdx.x; j < kAlignChunk; j += 256) {
+    const int i = i0 + j;
+    if (i < numel) atomicAdd(&hist[topk_ids[i]], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < num_experts; e += 256) chunk_hist[(size_t)blockIdx.x * num_experts + e] = hist[e];
+  const int nb = gridDim.x;
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < sorted_capacity; i += nb * 256) sorted_token_ids[i] = numel;
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < expert_capacity; i += nb * 256) {
+    expert_ids[i] = -1;
+    bucket_live[i] = 0;
+  }
+}
+
+// One workgroup of 512 threads, thread e = expert e.  chunk_hist[c][e] becomes the first slot of chunk c's
+// selections of expert e.
+__global__ void __launch_bounds__(512) k_align_offsets(const int* __restrict__ valid_tokens, int top_k, int num_experts,
+                                                        int block_size, int n_chunks_max, int expert_capacity,
+                                                        int* __restrict__ chunk_hist, int* __restrict__ expert_counts,
+                                                        int* __restrict__ expert_ids, int* __restrict__ bucket_live,
+                                                        int* __restrict__ num_tokens_post_pad) {
+  __shared__ int s_padded[kAlignMaxExperts];
+  __shared__ int s_base[kAlignMaxExperts + 1];
+  const int e = threadIdx.x;
+  const int numel = *valid_tokens * top_k;
+  const int n_chunks = min(n_chunks_max, (numel + kAlignChunk - 1) / kAlignChunk);
+  int count = 0;
+  if (e < num_experts)
+    for (int c = 0; c < n_chunks; ++c) count += chunk_hist[(size_t)c * num_experts + e];
+  if (e < kAlignMaxExperts) s_padded[e] = e < num_experts ? (count + block_size - 1) / block_size * block_size : 0;
+  __syncthreads();
+  if (e == 0) {
+    int acc = 0;
+    for (int i = 0; i < num_experts; ++i) {
+      s_base[i] = acc;
+      acc += s_padded[i];
+    }
+    s_base[num_experts] = acc;
+    *num_tokens_post_pad = acc;
+  }
+  __syncthreads();
+  if (e >= num_experts) return;
+  expert_counts[e] = count;
+  const int base = s_base[e];
+  int run = base;
+  for (int c = 0; c < n_chunks; ++c) {
+    const size_t i = (size_t)c * num_experts + e;
+    const int h = chunk_hist[i];
+    chunk_hist[i] = run;
+    run += h;
+  }
+  const int nblk = (count + block_size - 1) / block_size;
+  for (int b = 0; b < nblk; ++b) {
+    const int blk = base / block_size + b;
+    if (blk < expert_capacity) {
+      expert_ids[blk] = e;
+      bucket_live[blk] = min(block_size, count - b * block_size);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) k_align_place(const int* __restrict__ topk_ids, const int* __restrict__ valid_tokens,
+                                                      int top_k, int num_experts, int sorted_capacity,
+                                                      const int* __restrict__ chunk_first, int* __restrict__ sorted_token_ids) {
+  __shared__ int cnt[4][kAlignMaxExperts];  // next slot of expert e for wavefront w
+  const int numel = *valid_tokens * top_k;
+  const int i0 = blockIdx.x * kAlignChunk;
+  if (i0 >= numel) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // pass 1: per-wavefront counts
+  for (int e = threadIdx.x; e < 4 * kAlignMaxExperts; e += 256) (&cnt[0][0])[e] = 0;
+  __syncthreads();
+  int id[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int i = i0 + wave * 256 + r * 64 + lane;
+    id[r] = i < numel ? topk_ids[i] : -1;
+    if (id[r] >= 0) atomicAdd(&cnt[wave][id[r]], 1);
+  }
+  __syncthreads();
+  // counts -> first slots: this chunk's first slot of the expert, plus the earlier wavefronts' counts
+  for (int e = threadIdx.x; e < num_experts; e += 256) {
+    int run = chunk_first[(size_t)blockIdx.x * num_experts + e];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int h = cnt[w][e];
+      cnt[w][e] = run;
+      run += h;
+    }
+  }
+  __syncthreads();
+  // pass 2: rank among equals in index order, one distinct expert of the wavefront's 64 ids at a time
+  int* mine = cnt[wave];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int i = i0 + wave * 256 + r * 64 + lane;
+    const int v = id[r];
+    int pos = -1;
+    unsigned long long remaining = __ballot(v >= 0);
+    while (remaining) {
+      const int leader = __builtin_ctzll(remaining);
+      const int ev = __builtin_amdgcn_readlane(v, leader);
+      const unsigned long long same = __ballot(v == ev);
+      const int first = mine[ev];
+      if (v == ev) pos = first + __popcll(same & ((1ull << lane) - 1ull));
+      __builtin_amdgcn_wave_barrier();
+      if (lane == leader) mine[ev] = first + __popcll(same);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      remaining &= ~same;
+    }
+    if (pos >= 0 && pos < sorted_capacity) sorted_token_ids[pos] = i;
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // moe_reduce (crates/xabe-cuda/src/kernels/moe.rs:4049-4065): out[t] = sum_k partial[t*K+k], ascending k.
 // grid (max_tokens, ceil(hidden/256)).
 // ---------------------------------------------------------------------------------

@@ -124,7 +124,8 @@ def test_route_small_expert_counts(oracle, X):
         assert np.array_equal(ids[:9], oracle.route_batch(logits, K)[0].astype(np.int32)), (E, K)
 
 
-@pytest.mark.parametrize("tokens,max_tokens,block", [(37, 64, 32), (5, 8, 32), (200, 256, 32), (1500, 1536, 64)])
+@pytest.mark.parametrize("tokens,max_tokens,block", [(37, 64, 32), (5, 8, 32), (200, 256, 32), (1500, 1536, 64),
+                                                     (8192, 8192, 64), (700, 8192, 64), (1025, 2048, 64)])
 def test_dispatch_tables_are_exact(oracle, X, tokens, max_tokens, block):
     # moe_differential.rs:438-543: exact incl. padding, sentinel and -1 fill over the whole capacity
     r = oracle.Xorshift64Star(0xD15 + tokens)
@@ -160,6 +161,21 @@ def test_dispatch_collisions_all_tokens_one_expert(oracle, X):
     n = d.num_tokens_post_pad
     assert np.array_equal(b.sorted_token_ids().cpu().numpy()[:n], d.sorted_token_ids.astype(np.int32))
     assert np.array_equal(b.expert_ids().cpu().numpy()[: n // 32], d.expert_ids)
+
+
+def test_dispatch_collisions_at_prefill_width(oracle, X):
+    # the counting-sort form of the tables (8192 selections and up): every token to the same eight experts,
+    # so each expert's run spans every chunk and every wavefront of the placement
+    logits = np.zeros((3000, 256), np.float32)
+    logits[:, 100:108] = 5.0
+    k, b, g = _route(X, logits, 4096, 3000, block=64)
+    k.build_dispatch(b)
+    ids = b.topk_ids().cpu().numpy().reshape(4096, 8)[:3000]
+    d = oracle.moe_align_block_size(ids.astype(np.uint32), 64, 256)
+    n = d.num_tokens_post_pad
+    assert int(b.num_tokens_post_pad().cpu().numpy()[0]) == n
+    assert np.array_equal(b.sorted_token_ids().cpu().numpy()[:n], d.sorted_token_ids.astype(np.int32))
+    assert np.array_equal(b.expert_ids().cpu().numpy()[: n // 64], d.expert_ids)
 
 
 def test_geometry_and_error_paths(X):
