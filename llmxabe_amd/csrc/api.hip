@@ -743,6 +743,7 @@ int xabe_moe_router_logits(const xabe_moe_kernels* k, void* stream, const xabe_m
   }
   XABE_TRY(check_len("normed", g.max_tokens * g.hidden, normed_len));
   XABE_TRY(check_len("logits", g.max_tokens * g.num_experts, logits_len));
+  if (router_gemm_supported(k, fmt)) return launch_router_gemm(k, as_stream(stream), b, router, fmt, normed, logits);
   ExpertArgs a = base_args(k, b);
   a.w0 = static_cast<const uint8_t*>(router);
   a.x = normed;

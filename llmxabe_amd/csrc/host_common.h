@@ -61,6 +61,10 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
                         float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches = 7u);
 
 // matrix-core regime (mfma.hip)
+// router logits as an fp32 matrix-core GEMM at prefill widths (router_gemm.hip)
+bool router_gemm_supported(const xabe_moe_kernels* k, int router_quant);
+int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,
+                       int router_quant, const float* normed, float* logits);
 bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int gate_q, int up_q, int down_q, bool routed);
 int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
                                  xabe_quant_tensor up, xabe_quant_tensor down, const float* x);

@@ -1,0 +1,141 @@
+// Router logits at prefill widths: logits[t][e] = router[e] . normed[t] as a GEMM on the fp32 matrix
+// instruction (v_mfma_f32_32x32x2_f32).  The decode-style kernel re-reads the router once per two tokens
+// (8192 tokens: 4096 passes over it out of L2, 340 us); here a workgroup holds a 64-token x 128-expert tile
+// and walks the contraction in steps of 32, so the router is read once per 64 tokens.
+//
+// fp32 operands on purpose: the routing decision hangs on these numbers, and fp16 operands would move a few
+// selections per thousand tokens.  A Q8_0 router dequantises to exactly q * d in fp32 (the CPU reference's
+// value); products and sums are fp32 inside the matrix core.  The contraction order differs from the
+// decode kernels', so these logits agree with theirs to fp32 rounding, not bit for bit: as with the expert
+// contractions, a token is bit-identical across batches WITHIN a regime.
+// Replaces the reference's router launch for wide passes (crates/xabe-engine/src/block/moe.rs:1150-1184).
+#include <string.h>
+
+#include "device_common.h"
+#include "host_common.h"
+
+namespace xabe {
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int kRgM = 64;        // tokens per tile
+constexpr int kRgN = 128;       // experts per tile
+constexpr int kRgK = 32;        // contraction step: one Q8_0 block per row
+constexpr int kRgLdA = kRgM + 1;  // LDS tiles are k-major: element (k, m) at k * ld + m
+constexpr int kRgLdB = kRgN + 1;
+
+struct RouterGemmArgs {
+  const void* router;   // [E][H] f32, or Q8_0 blocks
+  const float* normed;  // [T][H]
+  float* logits;        // [T][E]
+  const int* valid_tokens;
+  int H, E;
+};
+
+// grid: (E / 128, ceil(max_tokens / 64)); 4 wavefronts as 2 (tokens) x 2 (experts), each 32 x 64.
+template <bool Q8>
+__global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
+  __shared__ float sA[kRgK * kRgLdA];
+  __shared__ float sB[kRgK * kRgLdB];
+  const int valid = *a.valid_tokens;
+  const int m0 = blockIdx.y * kRgM, n0 = blockIdx.x * kRgN;
+  if (m0 >= valid) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // A staging: thread -> (token row tid / 4, eight floats at (tid % 4) * 8); rows past the last live token
+  // re-read the last live one (computed, never stored)
+  const int am = tid >> 2, ak = (tid & 3) * 8;
+  const float* arow = a.normed + (size_t)min(m0 + am, valid - 1) * a.H + ak;
+  // B staging: thread -> (expert row tid / 2, sixteen elements at (tid % 2) * 16)
+  const int bn = tid >> 1, bk = (tid & 1) * 16;
+  const size_t brow_bytes = Q8 ? (size_t)(a.H / 32) * kQ8Bytes : (size_t)a.H * 4;
+  const uint8_t* brow = static_cast<const uint8_t*>(a.router) + (size_t)(n0 + bn) * brow_bytes;
+
+  float16v acc[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) acc[j] = (float16v)(0.0f);
+
+  const int nks = a.H / kRgK;
+  float4 ra[2];
+  float rb[16];
+  auto load_step = [&](int ks) {
+    ra[0] = reinterpret_cast<const float4*>(arow + (size_t)ks * kRgK)[0];
+    ra[1] = reinterpret_cast<const float4*>(arow + (size_t)ks * kRgK)[1];
+    if constexpr (Q8) {
+      // block ks of the row: d (fp16) then 32 codes; this thread takes codes bk .. bk + 15 (2-byte aligned)
+      const uint8_t* blk = brow + (size_t)ks * kQ8Bytes;
+      const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(blk));
+      const uint16_t* q = reinterpret_cast<const uint16_t*>(blk + 2 + bk);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t two = q[i];
+        rb[2 * i] = (float)(int8_t)(two & 0xff) * d;
+        rb[2 * i + 1] = (float)(int8_t)(two >> 8) * d;
+      }
+    } else {
+      const float4* p = reinterpret_cast<const float4*>(brow + ((size_t)ks * kRgK + bk) * 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 v = p[i];
+        rb[4 * i] = v.x; rb[4 * i + 1] = v.y; rb[4 * i + 2] = v.z; rb[4 * i + 3] = v.w;
+      }
+    }
+  };
+  load_step(0);
+  for (int ks = 0; ks < nks; ++ks) {
+    __syncthreads();  // the previous step's tiles have been read
+    const float va[8] = {ra[0].x, ra[0].y, ra[0].z, ra[0].w, ra[1].x, ra[1].y, ra[1].z, ra[1].w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sA[(ak + i) * kRgLdA + am] = va[i];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sB[(bk + i) * kRgLdB + bn] = rb[i];
+    __syncthreads();
+    if (ks + 1 < nks) load_step(ks + 1);  // in flight while the matrix core works
+    // operand layout of the 32x32x2 instruction: lane l supplies row (column) l % 32 at k = l / 32
+    const float* pa = &sA[(lane >> 5) * kRgLdA + wm * 32 + (lane & 31)];
+    const float* pb = &sB[(lane >> 5) * kRgLdB + wn * 64 + (lane & 31)];
+#pragma unroll
+    for (int kk = 0; kk < kRgK / 2; ++kk) {
+      const float av = pa[kk * 2 * kRgLdA];
+      const float b0 = pb[kk * 2 * kRgLdB], b1 = pb[kk * 2 * kRgLdB + 32];
+      acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[1], 0, 0, 0);
+    }
+  }
+  // acc[j][v]: tile row (v / 4) * 8 + (lane / 32) * 4 + v % 4, column lane % 32 of column block j
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int t = m0 + wm * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+    if (t >= valid) continue;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) a.logits[(size_t)t * a.E + n0 + wn * 64 + j * 32 + (lane & 31)] = acc[j][v];
+  }
+}
+
+bool router_gemm_supported(const xabe_moe_kernels* k, int router_quant) {
+  const xabe_moe_geometry& g = k->g;
+  // below ~2048 tokens the 64 x 128 tiles are too few to fill the chip and the decode-style kernel wins
+  if (!k->tensor_cores || k->exact_regime || k->force_community || g.max_tokens < 2048) return false;
+  if (!(router_quant < 0 || router_quant == XABE_QUANT_Q8_0)) return false;
+  return g.hidden % kRgK == 0 && g.num_experts % kRgN == 0;
+}
+
+int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,
+                       int router_quant, const float* normed, float* logits) {
+  const xabe_moe_geometry& g = k->g;
+  RouterGemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.router = router;
+  a.normed = normed;
+  a.logits = logits;
+  a.valid_tokens = b->valid_tokens;
+  a.H = (int)g.hidden;
+  a.E = (int)g.num_experts;
+  dim3 grid((unsigned)(g.num_experts / kRgN), (unsigned)((g.max_tokens + kRgM - 1) / kRgM));
+  if (router_quant < 0) hipLaunchKernelGGL(k_router_gemm<false>, grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(k_router_gemm<true>, grid, dim3(256), 0, s, a);
+  XABE_HIP_TRY(hipGetLastError());
+  return XABE_OK;
+}
+
+}  // namespace xabe

@@ -169,3 +169,29 @@ def test_prefill_rows_do_not_depend_on_batch_mates(oracle, X):
     la, lb = la.cpu().numpy(), lb.cpu().numpy()
     assert np.array_equal(la[77].view(np.uint32), lb[5].view(np.uint32))
     assert np.array_equal(la[5].view(np.uint32), lb[77].view(np.uint32))
+
+
+@pytest.mark.parametrize("router_q8", [True, False])
+def test_router_logits_matrix_core_path(oracle, X, router_q8):
+    # from 2048 tokens up the router runs on the fp32 matrix instruction: fp32 operands, so the logits agree
+    # with the CPU reference to fp32 reassociation (the decode-width kernel's bound), for live rows only
+    import torch
+
+    T, live = 2048, 1990
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
+    layer = make_layer(oracle, g, seed=715, router_q8=router_q8)
+    normed = activations(33, T, 2048, live)
+    k = X.MoeKernels(g)
+    b = k.buffers()
+    k.set_valid_tokens(b, live)
+    logits = torch.full((T, 256), 7.0, device="cuda")
+    d = layer.dev
+    k.router_logits(b, d.router, d.router_quant, normed, logits)
+    torch.cuda.synchronize()
+    got = logits.cpu().numpy()
+    assert np.all(got[live:] == 7.0)                                    # rows past the live tokens are not written
+    host = layer.host
+    w = (oracle.dequantize_row(oracle.Q8_0, host.router_q8) if router_q8 else host.router_f32).reshape(256, 2048)
+    rows = np.r_[0:40, 1000:1040, live - 40:live]
+    want = normed.cpu().numpy()[rows].astype(np.float64) @ w.astype(np.float64).T
+    assert rel_to_peak(got[rows], want) <= 2e-5
