@@ -185,6 +185,32 @@ def main() -> int:
                      for n, u, bts in zip(stage_names, stage_us, stage_bytes)],
     }
 
+    # ---- what this box can do, next to the nominal peaks: a plain device read and a plain fp16 GEMM,
+    # both library routines (nothing of this repository is in them)
+    with torch.cuda.stream(stream):
+        big = torch.ones(1 << 28, dtype=torch.int32, device="cuda")   # 1 GiB
+        big.sum()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(5):
+            big.sum()
+        e1.record(stream)
+        e1.synchronize()
+        read_gbps = 5 * big.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+        del big
+        ma = torch.randn(8192, 8192, device="cuda", dtype=torch.float16)
+        mb = torch.randn(8192, 8192, device="cuda", dtype=torch.float16)
+        torch.matmul(ma, mb)
+        e0.record(stream)
+        for _ in range(5):
+            torch.matmul(ma, mb)
+        e1.record(stream)
+        e1.synchronize()
+        gemm_tflops = 5 * 2 * 8192 ** 3 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+        del ma, mb
+    out["calibration"] = {"device_read_gbps": read_gbps, "device_read_what": "torch sum over 1 GiB of int32",
+                          "fp16_gemm_tflops": gemm_tflops, "fp16_gemm_what": "torch.matmul 8192^3 fp16 (hipBLASLt)"}
+
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(layers[0], g, x, T, args.cpu_seconds)
     print(json.dumps(out))
