@@ -148,6 +148,30 @@ static bool launch_block_resident(Shape shape, const ExpertArgs& a, size_t units
   return true;
 }
 
+// Rows longer than one step, no expert indirection (dense sibling, wide shared experts): the step-outer
+// kernel, R rows per wavefront (2 for a gate/up pair, 4 for one matrix).  `la.norm_w` set: normalise on
+// load; `la.l_out` set: add the residual in the epilogue.
+bool launch_long_rows(const xabe_moe_kernels* k, int quant, int nm, const LongRowArgs& la, hipStream_t s) {
+  const ExpertArgs& a = la.m;
+  if (k->force_community || a.K <= 2048 || !(quant == XABE_QUANT_Q6K || quant == XABE_QUANT_Q8_0)) return false;
+  const int r = nm == 2 ? 2 : 4;
+  if (a.n_rows % (kWavesPerWg * r) != 0 || a.n_rows / (kWavesPerWg * r) > 65535) return false;
+  if ((la.norm_w != nullptr) != (nm == 2) && la.norm_w) return false;  // normalising only feeds gate/up
+  dim3 grid((unsigned)(a.n_rows / (kWavesPerWg * r)), (unsigned)((k->g.max_tokens + 7) / 8));
+  const bool norm = la.norm_w != nullptr, resid = la.l_out != nullptr;
+#define XABE_LONG(Q)                                                                                                   \
+  do {                                                                                                                 \
+    if (nm == 2 && norm) hipLaunchKernelGGL((k_shared_long_rows<Q, 2, 2, kXNorm, false>), grid, dim3(256), 0, s, la);  \
+    else if (nm == 2) hipLaunchKernelGGL((k_shared_long_rows<Q, 2, 2, kXPlain, false>), grid, dim3(256), 0, s, la);    \
+    else if (resid) hipLaunchKernelGGL((k_shared_long_rows<Q, 1, 4, kXPlain, true>), grid, dim3(256), 0, s, la);       \
+    else hipLaunchKernelGGL((k_shared_long_rows<Q, 1, 4, kXPlain, false>), grid, dim3(256), 0, s, la);                 \
+  } while (0)
+  if (quant == XABE_QUANT_Q6K) XABE_LONG(kQ6K);
+  else XABE_LONG(kQ8_0);
+#undef XABE_LONG
+  return true;
+}
+
 int pick_tile_rows(const xabe_moe_kernels* k, size_t live_units, int n_rows, int rps) {
   // aim for ~12 wavefronts per CU across the launch
   const size_t items = std::max<size_t>(1, live_units) * (size_t)n_rows / rps;
@@ -169,6 +193,15 @@ static int launch_expert(const xabe_moe_kernels* k, Mode mode, int quant, int nm
     if (quant == XABE_QUANT_Q6K) done = nm == 2 ? launch_block_resident<kQ6K, 2>(shape, a, units, s) : launch_block_resident<kQ6K, 1>(shape, a, units, s);
     else if (quant == XABE_QUANT_Q8_0) done = nm == 2 ? launch_block_resident<kQ8_0, 2>(shape, a, units, s) : launch_block_resident<kQ8_0, 1>(shape, a, units, s);
     if (done) {
+      XABE_HIP_TRY(hipGetLastError());
+      return XABE_OK;
+    }
+  }
+  if (mode == kShared && a.expert_bytes == 0) {
+    LongRowArgs la;
+    memset(&la, 0, sizeof(la));
+    la.m = a;
+    if (launch_long_rows(k, quant, nm, la, s)) {
       XABE_HIP_TRY(hipGetLastError());
       return XABE_OK;
     }
@@ -627,6 +660,53 @@ static int shared_fp32(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffer
   a.K = (int)g.intermediate;
   a.n_rows = (int)g.hidden;
   XABE_TRY(launch_expert(k, kShared, down.quant, 1, a, units, units, s));
+  return XABE_OK;
+}
+
+// The dense block's fp32 path on the long-row kernel, the residual folded into down: three launches.
+// Returns false (nothing launched) where the long-row kernel does not apply.
+static int check_shared_stacks(const xabe_moe_kernels* k, xabe_quant_tensor gate, xabe_quant_tensor up,
+                               xabe_quant_tensor down);
+
+int xabe::dense_fp32_fused(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                           xabe_quant_tensor up, xabe_quant_tensor down, const float* post_norm, float eps,
+                           const float* residual, float* normed, float* ffn_out, float* l_out, bool* launched) {
+  const xabe_moe_geometry& g = k->g;
+  *launched = false;
+  XABE_TRY(check_shared_stacks(k, gate, up, down));  // the checks xabe_moe_shared_expert makes
+  LongRowArgs la;
+  memset(&la, 0, sizeof(la));
+  la.m = base_args(k, b);
+  la.m.w0 = static_cast<const uint8_t*>(gate.bytes);
+  la.m.w1 = static_cast<const uint8_t*>(up.bytes);
+  // (normalising on load is there in the kernel, but with thousands of wavefronts each re-deriving the
+  // RMS scale of every token it costs more than the stand-alone RMSNorm launch it saves: measured)
+  XABE_TRY(xabe_rms_norm(s, residual, g.max_tokens * g.hidden, post_norm, g.hidden, normed, g.max_tokens * g.hidden,
+                         g.max_tokens, g.hidden, eps));
+  la.m.x = normed;
+  la.m.out = b->shared_inter;
+  la.m.K = (int)g.hidden;
+  la.m.n_rows = (int)g.intermediate;
+  LongRowArgs ld;
+  memset(&ld, 0, sizeof(ld));
+  ld.m = base_args(k, b);
+  ld.m.w0 = static_cast<const uint8_t*>(down.bytes);
+  ld.m.x = b->shared_inter;
+  ld.m.out = ffn_out;
+  ld.m.K = (int)g.intermediate;
+  ld.m.n_rows = (int)g.hidden;
+  ld.residual = residual;
+  ld.l_out = l_out;
+  // both or neither: check the second shape before launching the first
+  const int r_up = 2, r_down = 4;
+  if (k->force_community || g.hidden <= 2048 || g.intermediate <= 2048) return XABE_OK;
+  if (g.intermediate % (kWavesPerWg * r_up) != 0 || g.hidden % (kWavesPerWg * r_down) != 0) return XABE_OK;
+  auto ok = [](int q) { return q == XABE_QUANT_Q6K || q == XABE_QUANT_Q8_0; };
+  if (!ok(gate.quant) || !ok(down.quant)) return XABE_OK;
+  if (!launch_long_rows(k, gate.quant, 2, la, s) || !launch_long_rows(k, down.quant, 1, ld, s))
+    return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "dense block: the long-row kernel refused a shape it was checked for");
+  XABE_HIP_TRY(hipGetLastError());
+  *launched = true;
   return XABE_OK;
 }
 

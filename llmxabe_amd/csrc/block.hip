@@ -226,10 +226,17 @@ int xabe_dense_ffn_block_forward(xabe_dense_ffn_block* blk, void* stream, const 
   XABE_TRY(blk_check_len("ffn_out", blk->n_act, ffn_out_len));
   XABE_TRY(blk_check_len("l_out", blk->n_act, l_out_len));
   XABE_TRY(xabe_moe_set_valid_tokens(blk->moe, stream, blk->buffers, tokens));
-  XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
-                         g.hidden, blk->eps));
   const bool wide = g.max_tokens >= kMfmaMinTokens && xabe_moe_kernels_tensor_cores_enabled(blk->moe) &&
                     mfma_supported(blk->moe, blk->buffers, w->gate.quant, w->up.quant, w->down.quant, false);
+  // fp32 widths: norm folded into gate/up, residual into down (same values, two launches instead of four)
+  if (!wide && w->post_norm) {
+    bool launched = false;
+    XABE_TRY(dense_fp32_fused(blk->moe, as_stream(stream), blk->buffers, w->gate, w->up, w->down, w->post_norm, blk->eps,
+                              residual, blk->normed, ffn_out, l_out, &launched));
+    if (launched) return XABE_OK;
+  }
+  XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
+                         g.hidden, blk->eps));
   if (wide)
     XABE_TRY(xabe_moe_shared_expert_mma(blk->moe, stream, blk->buffers, w->gate, w->up, w->down, blk->normed, blk->n_act,
                                         ffn_out, blk->n_act));

@@ -498,6 +498,124 @@ __device__ __forceinline__ void shared_body(const ExpertArgs& a, int chunk, int 
   }
 }
 
+// Shared expert / dense MLP with rows longer than one step (the dense sibling: 5120 and 17408 elements).
+// A wavefront owns R rows and walks the contraction step by step with the rows inside: the step's weights
+// for all R rows are requested together, the step's activations are read
+// once per step instead of once per (row, step), and up to eight tokens run against the same registers, so
+// the weights are read once per eight tokens instead of once per two.  Per (row, token) the lane partial
+// still accumulates step after step and is reduced once at the end: the operation order of matvec_rows'
+// long-row path, so the bits are the same.  grid (n_rows / (4 R), ceil(max_tokens / 8)).
+//   XMODE = kXNorm: `a.x` holds the un-normalised rows; they are RMS-normalised on load (and the workgroups
+//           of row tile 0 write the normalised rows to `normed_out`): the stand-alone RMSNorm's bits.
+//   RESID:  also write l_out = out + residual (the dense block's last step).
+struct LongRowArgs {
+  ExpertArgs m;
+  const float* norm_w;    // kXNorm
+  float* normed_out;      // kXNorm, may be null
+  const float* residual;  // RESID
+  float* l_out;           // RESID
+  float eps;
+};
+
+template <int QUANT, int NM, int R, int XMODE, bool RESID>
+__global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
+  using F = Fmt<QUANT>;
+  using Raw = typename F::Raw;
+  constexpr int kTok = 8;
+  const ExpertArgs& a = la.m;
+  const int valid = *a.valid_tokens;
+  const int t0 = blockIdx.y * kTok;
+  if (t0 >= valid) return;
+  const int nt = min(kTok, valid - t0);
+  const LaneGeom g = lane_geom<QUANT>();
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int row0 = ((int)blockIdx.x * kWavesPerWg + wave) * R;
+  const size_t row_bytes = (size_t)(a.K / F::kBlockElems) * F::kBlockBytes;
+  const int steps = (a.K + kStepElems - 1) / kStepElems;
+  auto load_step = [&](int k, Raw (&raw)[R][NM]) {
+    const bool act = lane_koff<QUANT, 1>(g, k) < a.K;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const size_t off = (size_t)(row0 + r) * row_bytes + (size_t)k * F::kChunkBytes;
+      load_raw<QUANT>(a.w0 + off, act, g, raw[r][0]);
+      if constexpr (NM == 2) load_raw<QUANT>(a.w1 + off, act, g, raw[r][NM - 1]);
+    }
+  };
+  Raw raw[R][NM];
+  float inv[kTok];
+#pragma unroll
+  for (int t = 0; t < kTok; ++t) inv[t] = 1.0f;
+  if constexpr (XMODE == kXNorm) {
+#pragma unroll
+    for (int t = 0; t < kTok; ++t)
+      if (t < nt) inv[t] = row_inv_rms(a.x + (size_t)(t0 + t) * a.K, a.K, la.eps);
+    if (blockIdx.x == 0 && la.normed_out) {
+      for (int t = 0; t < nt; ++t) {
+        const float* xr = a.x + (size_t)(t0 + t) * a.K;
+        const float it = t == 0 ? inv[0] : t == 1 ? inv[1] : t == 2 ? inv[2] : t == 3 ? inv[3] : t == 4 ? inv[4] : t == 5 ? inv[5] : t == 6 ? inv[6] : inv[7];
+        for (int j = threadIdx.x; j < a.K; j += 256) la.normed_out[(size_t)(t0 + t) * a.K + j] = xr[j] * it * la.norm_w[j];
+      }
+    }
+  }
+  float acc[R][NM][kTok];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+      for (int t = 0; t < kTok; ++t) acc[r][m][t] = 0.0f;
+  for (int k = 0; k < steps; ++k) {
+    const int koff = lane_koff<QUANT, 1>(g, k);
+    const bool act = koff < a.K;
+    load_step(k, raw);
+#pragma unroll
+    for (int c = 0; c < kTok / 2; ++c) {
+      if (2 * c >= nt) break;
+      if (2 * c + 1 < nt) {
+        float x[2][32], xs[2][4];
+        load_x<QUANT, XMODE>(a.x + (size_t)(t0 + 2 * c) * a.K, koff, act, g, x[0], xs[0], XNorm{inv[2 * c], la.norm_w});
+        load_x<QUANT, XMODE>(a.x + (size_t)(t0 + 2 * c + 1) * a.K, koff, act, g, x[1], xs[1], XNorm{inv[2 * c + 1], la.norm_w});
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int m = 0; m < NM; ++m) {
+            float tt[2] = {acc[r][m][2 * c], acc[r][m][2 * c + 1]};
+            accum<QUANT, 2>(raw[r][m], g, x, xs, tt);
+            acc[r][m][2 * c] = tt[0];
+            acc[r][m][2 * c + 1] = tt[1];
+          }
+      } else {
+        float x[1][32], xs[1][4];
+        load_x<QUANT, XMODE>(a.x + (size_t)(t0 + 2 * c) * a.K, koff, act, g, x[0], xs[0], XNorm{inv[2 * c], la.norm_w});
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int m = 0; m < NM; ++m) {
+            float tt[1] = {acc[r][m][2 * c]};
+            accum<QUANT, 1>(raw[r][m], g, x, xs, tt);
+            acc[r][m][2 * c] = tt[0];
+          }
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < kTok; ++t) {
+    if (t >= nt) break;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float tot[NM];
+#pragma unroll
+      for (int m = 0; m < NM; ++m) tot[m] = group_sum<64>(acc[r][m][t]);
+      if (g.lane == 0) {
+        const size_t i = (size_t)(t0 + t) * a.n_rows + row0 + r;
+        const float v = NM == 2 ? silu_f(tot[0]) * tot[NM - 1] : 1.0f * tot[0];
+        a.out[i] = v;
+        if constexpr (RESID) la.l_out[i] = v + la.residual[i];
+      }
+    }
+  }
+}
+
 template <int QUANT, int KS, int RPS, int NM>
 __global__ void __launch_bounds__(256) k_expert_shared(ExpertArgs a) {
   shared_body<QUANT, KS, RPS, NM>(a, blockIdx.y, blockIdx.x);

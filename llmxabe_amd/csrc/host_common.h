@@ -61,6 +61,11 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
                         float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches = 7u);
 
 // matrix-core regime (mfma.hip)
+// dense block, fp32 widths, rows longer than one step: norm + gate/up, down + residual (api.hip)
+// (`*launched` false and XABE_OK: not applicable, nothing launched)
+int dense_fp32_fused(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
+                     xabe_quant_tensor up, xabe_quant_tensor down, const float* post_norm, float eps,
+                     const float* residual, float* normed, float* ffn_out, float* l_out, bool* launched);
 // router logits as an fp32 matrix-core GEMM at prefill widths (router_gemm.hip)
 bool router_gemm_supported(const xabe_moe_kernels* k, int router_quant);
 int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,

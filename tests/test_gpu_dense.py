@@ -85,3 +85,26 @@ def test_dense_prefill_2048_matches_oracle_on_sampled_rows(oracle, dense):
     x2, ffn2, _, _ = _run(X, w, H, I, 64, 2, seed=53, disable_mfma=True)
     _, f2, _ = oracle.dense_block_forward(H, I, 1e-6, host["pn"], host["g"], host["u"], host["d"], x2[:2], threads=16)
     assert rel_to_peak(ffn2[:2], f2) <= DECODE_REL
+
+
+@pytest.mark.parametrize("max_tokens,tokens", [(1, 1), (8, 8), (16, 13)])
+def test_long_row_kernel_equals_the_plain_one(dense, max_tokens, tokens):
+    # rows longer than one 2048-element step take the step-outer kernel (weights read once per eight tokens);
+    # force_community keeps the row-outer streaming kernel: same operation order per (row, token), same bits
+    import torch
+
+    X, w, host, H, I = dense
+    g = X.MoeGeometry(1, 1, H, I, X.moe_block_size(max_tokens), max_tokens)
+    x = X.synth_normal_f32(77, max_tokens * H, 1.0).view(max_tokens, H)
+    outs = []
+    for plain in (False, True):
+        k = X.MoeKernels(g)
+        k.force_community(plain)
+        b = k.shared_only_buffers(False)
+        k.set_valid_tokens(b, tokens)
+        out = torch.zeros(max_tokens, H, device="cuda")
+        k.shared_expert(b, w.gate, w.up, w.down, x, out)
+        torch.cuda.synchronize()
+        outs.append(out.cpu().numpy().copy())
+    assert outs[0][:tokens].any() and not outs[0][tokens:].any()
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
