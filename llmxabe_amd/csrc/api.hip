@@ -149,26 +149,54 @@ static bool launch_block_resident(Shape shape, const ExpertArgs& a, size_t units
 }
 
 // Rows longer than one step, no expert indirection (dense sibling, wide shared experts): the step-outer
-// kernel, R rows per wavefront (2 for a gate/up pair, 4 for one matrix).  `la.norm_w` set: normalise on
-// load; `la.l_out` set: add the residual in the epilogue.
+// kernel, R rows per wavefront (2 for a gate/up pair, 4 for one matrix).  `la.l_out` set: add the residual
+// in the epilogue.
 bool launch_long_rows(const xabe_moe_kernels* k, int quant, int nm, const LongRowArgs& la, hipStream_t s) {
   const ExpertArgs& a = la.m;
   if (k->force_community || a.K <= 2048 || !(quant == XABE_QUANT_Q6K || quant == XABE_QUANT_Q8_0)) return false;
+  // rows per wavefront: 2 gate/up pairs or 4 single rows (the step's activations are read once for all of
+  // them).  Wavefronts are independent, so a matrix with few row groups is launched as one-wavefront
+  // workgroups, which spread evenly over the CUs.
+  const int tok = k->g.max_tokens == 1 ? 1 : 2;  // tokens per pass over the weights
   const int r = nm == 2 ? 2 : 4;
-  if (a.n_rows % (kWavesPerWg * r) != 0 || a.n_rows / (kWavesPerWg * r) > 65535) return false;
-  if ((la.norm_w != nullptr) != (nm == 2) && la.norm_w) return false;  // normalising only feeds gate/up
-  dim3 grid((unsigned)(a.n_rows / (kWavesPerWg * r)), (unsigned)((k->g.max_tokens + 7) / 8));
-  const bool norm = la.norm_w != nullptr, resid = la.l_out != nullptr;
-#define XABE_LONG(Q)                                                                                                   \
-  do {                                                                                                                 \
-    if (nm == 2 && norm) hipLaunchKernelGGL((k_shared_long_rows<Q, 2, 2, kXNorm, false>), grid, dim3(256), 0, s, la);  \
-    else if (nm == 2) hipLaunchKernelGGL((k_shared_long_rows<Q, 2, 2, kXPlain, false>), grid, dim3(256), 0, s, la);    \
-    else if (resid) hipLaunchKernelGGL((k_shared_long_rows<Q, 1, 4, kXPlain, true>), grid, dim3(256), 0, s, la);       \
-    else hipLaunchKernelGGL((k_shared_long_rows<Q, 1, 4, kXPlain, false>), grid, dim3(256), 0, s, la);                 \
+  if (a.n_rows % (kWavesPerWg * r) != 0) return false;
+  const unsigned passes = (unsigned)((k->g.max_tokens + tok - 1) / tok);
+  const int groups = a.n_rows / r;
+  const unsigned waves = (size_t)groups / kWavesPerWg * passes < (size_t)4 * k->num_cus ? 1 : kWavesPerWg;
+  if (groups / waves > 0x7fffffffu / 64) return false;
+  dim3 grid((unsigned)groups / waves, passes), block(64 * waves);
+  const bool resid = la.l_out != nullptr;
+  // the coalesced loader reads whole 16-byte pieces: the tensors must start and end on 16-byte boundaries
+  const size_t row_bytes = (size_t)a.K / xabe_expert_quant_block_elements(quant) * xabe_expert_quant_block_bytes(quant);
+  auto on16 = [&](const uint8_t* w) { return !w || (reinterpret_cast<uintptr_t>(w) % 16 == 0 && ((size_t)a.n_rows * row_bytes) % 16 == 0); };
+  const bool staged = on16(a.w0) && on16(a.w1);
+#define XABE_LONG4(Q, ST, TOK, R)                                                                                    \
+  do {                                                                                                                \
+    if (nm == 2) hipLaunchKernelGGL((k_shared_long_rows<Q, 2, R, TOK, false, ST>), grid, block, 0, s, la);            \
+    else if (resid) hipLaunchKernelGGL((k_shared_long_rows<Q, 1, R, TOK, true, ST>), grid, block, 0, s, la);          \
+    else hipLaunchKernelGGL((k_shared_long_rows<Q, 1, R, TOK, false, ST>), grid, block, 0, s, la);                \
+  } while (0)
+#define XABE_LONG3(Q, ST, TOK)                              \
+  do {                                                      \
+    if (nm == 2) XABE_LONG4(Q, ST, TOK, 2);                 \
+    else XABE_LONG4(Q, ST, TOK, 4);                         \
+  } while (0)
+#define XABE_LONG2(Q, ST)                 \
+  do {                                    \
+    if (tok == 1) XABE_LONG3(Q, ST, 1);   \
+    else XABE_LONG3(Q, ST, 2);            \
+  } while (0)
+#define XABE_LONG(Q)                      \
+  do {                                    \
+    if (staged) XABE_LONG2(Q, true);      \
+    else XABE_LONG2(Q, false);            \
   } while (0)
   if (quant == XABE_QUANT_Q6K) XABE_LONG(kQ6K);
   else XABE_LONG(kQ8_0);
+#undef XABE_LONG4
+#undef XABE_LONG3
 #undef XABE_LONG
+#undef XABE_LONG2
   return true;
 }
 
@@ -679,8 +707,8 @@ int xabe::dense_fp32_fused(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_bu
   la.m = base_args(k, b);
   la.m.w0 = static_cast<const uint8_t*>(gate.bytes);
   la.m.w1 = static_cast<const uint8_t*>(up.bytes);
-  // (normalising on load is there in the kernel, but with thousands of wavefronts each re-deriving the
-  // RMS scale of every token it costs more than the stand-alone RMSNorm launch it saves: measured)
+  // (normalising on load was tried: with thousands of wavefronts each re-deriving the RMS scale of every
+  // token it costs more than the stand-alone RMSNorm launch it saves)
   XABE_TRY(xabe_rms_norm(s, residual, g.max_tokens * g.hidden, post_norm, g.hidden, normed, g.max_tokens * g.hidden,
                          g.max_tokens, g.hidden, eps));
   la.m.x = normed;
@@ -798,6 +826,8 @@ int xabe_rms_norm(void* stream, const float* x, size_t x_len, const float* weigh
   XABE_TRY(check_len("out", rows * width, out_len));
   if (rows == 0 || width == 0) return XABE_OK;
   if (width % 4 != 0) return set_error(XABE_ERR_INVALID_ARGUMENT, "rms_norm: width %zu is not a multiple of 4", width);
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out)) % 16 != 0)
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "rms_norm: x, weight and out must be 16-byte aligned");
   hipLaunchKernelGGL(k_rms_norm_rows, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), x, weight, out, (int)width, eps);
   XABE_HIP_TRY(hipGetLastError());
   return XABE_OK;

@@ -75,31 +75,6 @@ struct DecodeArgs {
   int tiles_r, tiles_s, tiles_g, tiles_d;  // row tiles: router, shared gate/up (launch A), gate/up (B), down (C)
 };
 
-// The lane's 32 activations of one step from a row in global memory or LDS, raw.
-template <int QUANT>
-__device__ __forceinline__ void lane_x_load(const float* row, int koff, const LaneGeom& g, float (&v)[32]) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int off = QUANT == kQ6K ? koff + g.half * 128 + j * 32 + g.l8 * 8 : koff + j * 8;
-    const float4 a = reinterpret_cast<const float4*>(row + off)[0];
-    const float4 b = reinterpret_cast<const float4*>(row + off)[1];
-    v[j * 8 + 0] = a.x; v[j * 8 + 1] = a.y; v[j * 8 + 2] = a.z; v[j * 8 + 3] = a.w;
-    v[j * 8 + 4] = b.x; v[j * 8 + 5] = b.y; v[j * 8 + 6] = b.z; v[j * 8 + 7] = b.w;
-  }
-}
-
-// xs[j] = -32 * (sum of the j-th eight), the Q6_K code offset folded out of the inner loop (as load_x).
-template <int QUANT>
-__device__ __forceinline__ void lane_x_offsets(const float (&x)[32], float (&xs)[4]) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    float s = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) s += x[j * 8 + i];
-    xs[j] = QUANT == kQ6K ? -32.0f * s : 0.0f;
-  }
-}
-
 // One step (RPS rows of K = 2048 / RPS elements) of a matrix, or of a gate/up pair, against TC tokens whose
 // rows are normalised on load.  Issues every load before the first use.
 //   NM = 2: out[t][row] = silu(gate . x_t) * (up . x_t);   NM = 1: out[t][row] = (w . x_t) (+ bias[row]).

@@ -14,6 +14,8 @@
 // decodes to the same bits alone or in a batch (tests/test_gpu_batch_invariance.py).
 #pragma once
 
+#include <type_traits>
+
 #include "device_common.h"
 
 namespace xabe {
@@ -181,6 +183,71 @@ __device__ __forceinline__ void accum(const typename Fmt<QUANT>::Raw& r, const L
   if constexpr (QUANT == kQ6K) q6_accum<TC>(r, g.l8, x, xs, tot);
   else if constexpr (QUANT == kQ8_0) q8_accum<TC>(r, x, tot);
   else f32_accum<TC>(r, x, tot);
+}
+
+// ---------------------------------------------------------------------------------
+// Coalesced form of load_raw.  A lane picking its own fields out of global memory touches every cache
+// line of the step with every one of its seven to ten load instructions, and the vector L1 serves a
+// line that is still pending by stalling; measured on this part, that halves the streaming rate
+// (2.7 against 5.5 TB/s).  Instead the wavefront requests the step as consecutive 16-byte pieces (each
+// line touched once), parks them in a wavefront-private LDS slot and picks the fields up from there with
+// the same funnel loads, so the Raw it produces is bit for bit the one load_raw produces.
+//   stage_load:  issue the global loads of one step (`nbytes` live bytes starting at `chunk`, any 2-byte
+//                alignment).  The 16-byte window around them must lie inside the tensor: the host checks
+//                that the tensor starts and ends on 16-byte boundaries.
+//   stage_pick:  pieces -> LDS slot -> Raw.  Slots are private to a wavefront, whose LDS operations
+//                complete in program order; the fences only keep the compiler from reordering them.
+// ---------------------------------------------------------------------------------
+template <int QUANT>
+struct StageFmt;
+template <>
+struct StageFmt<kQ6K> {
+  static constexpr int kPieces = 2;        // 1680 (+14) bytes: up to 106 pieces
+  static constexpr int kSlotBytes = 1696;
+};
+template <>
+struct StageFmt<kQ8_0> {
+  static constexpr int kPieces = 3;        // 2176 (+14) bytes: up to 137 pieces
+  static constexpr int kSlotBytes = 2192;
+};
+
+typedef uint32_t stage_piece __attribute__((ext_vector_type(4)));  // a first-class vector: stays in registers
+
+template <int QUANT>
+struct Staged {
+  stage_piece p[StageFmt<QUANT>::kPieces];
+  uint32_t mis;  // bytes from the 16-byte boundary below `chunk` to `chunk`
+  int last;      // index of the last live piece
+};
+
+template <int QUANT>
+__device__ __forceinline__ void stage_load(const uint8_t* chunk, uint32_t nbytes, Staged<QUANT>& s) {
+  s.mis = (uint32_t)(reinterpret_cast<uintptr_t>(chunk) & 15u);
+  s.last = (int)((s.mis + nbytes + 15u) >> 4) - 1;
+  const stage_piece* base = reinterpret_cast<const stage_piece*>(chunk - s.mis);
+  const int lane = (int)__lane_id();
+#pragma unroll
+  for (int i = 0; i < StageFmt<QUANT>::kPieces; ++i) s.p[i] = base[min(lane + 64 * i, s.last)];
+}
+
+template <int QUANT>
+__device__ __forceinline__ void stage_pick(const Staged<QUANT>& s, uint8_t* slot, bool active, const LaneGeom& g,
+                                           typename Fmt<QUANT>::Raw& r) {
+  const int lane = (int)__lane_id();
+#pragma unroll
+  for (int i = 0; i < StageFmt<QUANT>::kPieces; ++i)  // lanes past the last piece repeat its store
+    reinterpret_cast<stage_piece*>(slot)[min(lane + 64 * i, s.last)] = s.p[i];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (active) {
+    if constexpr (QUANT == kQ6K) q6_load(slot, g.lane_off + s.mis, g.half, g.l8, r);
+    else q8_load(slot, g.lane_off + s.mis, r);
+  } else {
+    raw_zero<QUANT>(r);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
 }
 
 // ---------------------------------------------------------------------------------
@@ -498,119 +565,152 @@ __device__ __forceinline__ void shared_body(const ExpertArgs& a, int chunk, int 
   }
 }
 
+// The lane's 32 activations of one step from a row in global memory or LDS, raw (no arithmetic, so a
+// caller can request them and other data together and do the arithmetic when they arrive).
+template <int QUANT>
+__device__ __forceinline__ void lane_x_load(const float* row, int koff, const LaneGeom& g, float (&v)[32]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int off = QUANT == kQ6K ? koff + g.half * 128 + j * 32 + g.l8 * 8 : koff + j * 8;
+    const float4 a = reinterpret_cast<const float4*>(row + off)[0];
+    const float4 b = reinterpret_cast<const float4*>(row + off)[1];
+    v[j * 8 + 0] = a.x; v[j * 8 + 1] = a.y; v[j * 8 + 2] = a.z; v[j * 8 + 3] = a.w;
+    v[j * 8 + 4] = b.x; v[j * 8 + 5] = b.y; v[j * 8 + 6] = b.z; v[j * 8 + 7] = b.w;
+  }
+}
+
+// xs[j] = -32 * (sum of the j-th eight), the Q6_K code offset folded out of the inner loop (as load_x).
+template <int QUANT>
+__device__ __forceinline__ void lane_x_offsets(const float (&x)[32], float (&xs)[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += x[j * 8 + i];
+    xs[j] = QUANT == kQ6K ? -32.0f * s : 0.0f;
+  }
+}
+
+// Everything above this point in program order has been issued before anything below it is: keeps the
+// compiler from sinking a batch of loads down to their first uses, which would serialise them.
+__device__ __forceinline__ void issue_fence() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 // Shared expert / dense MLP with rows longer than one step (the dense sibling: 5120 and 17408 elements).
-// A wavefront owns R rows and walks the contraction step by step with the rows inside: the step's weights
-// for all R rows are requested together, the step's activations are read
-// once per step instead of once per (row, step), and up to eight tokens run against the same registers, so
-// the weights are read once per eight tokens instead of once per two.  Per (row, token) the lane partial
-// still accumulates step after step and is reduced once at the end: the operation order of matvec_rows'
-// long-row path, so the bits are the same.  grid (n_rows / (4 R), ceil(max_tokens / 8)).
-//   XMODE = kXNorm: `a.x` holds the un-normalised rows; they are RMS-normalised on load (and the workgroups
-//           of row tile 0 write the normalised rows to `normed_out`): the stand-alone RMSNorm's bits.
+// A wavefront owns R rows at a time and walks the contraction step by step with the rows inside: the step's
+// weights for all R rows are requested together and the step's activations are read once per step instead
+// of once per (row, step).  Per (row, token) the lane partial accumulates step after step and is reduced
+// once at the end: the operation order of matvec_rows' long-row path, so the bits are the same.
+// grid (row groups / wavefronts per workgroup; ceil(max_tokens / TOK)), TOK = 1 or 2 tokens per pass over
+// the weights (later passes find most of them in the memory-side cache); 64 or 256 threads.
+//   Software pipeline: the next step's weights are requested before this step's accumulation and its
+//   activations right after it, into the registers the accumulation has just released.
+//   STAGED: weights through the coalesced loader (stage_load / stage_pick); otherwise per-lane field loads.
 //   RESID:  also write l_out = out + residual (the dense block's last step).
 struct LongRowArgs {
   ExpertArgs m;
-  const float* norm_w;    // kXNorm
-  float* normed_out;      // kXNorm, may be null
   const float* residual;  // RESID
   float* l_out;           // RESID
-  float eps;
 };
 
-template <int QUANT, int NM, int R, int XMODE, bool RESID>
+template <int QUANT, int NM, int R, int TOK, bool RESID, bool STAGED>
 __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
   using F = Fmt<QUANT>;
   using Raw = typename F::Raw;
-  constexpr int kTok = 8;
+  using Pending = typename std::conditional<STAGED, Staged<QUANT>, Raw>::type;
+  constexpr int kSlot = StageFmt<QUANT>::kSlotBytes;
+  __shared__ __attribute__((aligned(16))) uint8_t s_slots[STAGED ? kWavesPerWg * R * NM * kSlot : 16];
   const ExpertArgs& a = la.m;
   const int valid = *a.valid_tokens;
-  const int t0 = blockIdx.y * kTok;
+  const int t0 = blockIdx.y * TOK;
   if (t0 >= valid) return;
-  const int nt = min(kTok, valid - t0);
+  const int nt = min(TOK, valid - t0);
   const LaneGeom g = lane_geom<QUANT>();
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const int row0 = ((int)blockIdx.x * kWavesPerWg + wave) * R;
   const size_t row_bytes = (size_t)(a.K / F::kBlockElems) * F::kBlockBytes;
   const int steps = (a.K + kStepElems - 1) / kStepElems;
-  auto load_step = [&](int k, Raw (&raw)[R][NM]) {
-    const bool act = lane_koff<QUANT, 1>(g, k) < a.K;
+  const int wg_waves = (int)(blockDim.x >> 6);  // 4, or 1 for a matrix with few row groups
+#pragma unroll 1
+  for (int rg = (int)blockIdx.x * wg_waves + wave; rg < a.n_rows / R; rg += (int)gridDim.x * wg_waves) {
+    const int row0 = rg * R;
+    float acc[R][NM][TOK];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const size_t off = (size_t)(row0 + r) * row_bytes + (size_t)k * F::kChunkBytes;
-      load_raw<QUANT>(a.w0 + off, act, g, raw[r][0]);
-      if constexpr (NM == 2) load_raw<QUANT>(a.w1 + off, act, g, raw[r][NM - 1]);
-    }
-  };
-  Raw raw[R][NM];
-  float inv[kTok];
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-  for (int t = 0; t < kTok; ++t) inv[t] = 1.0f;
-  if constexpr (XMODE == kXNorm) {
+      for (int m = 0; m < NM; ++m)
 #pragma unroll
-    for (int t = 0; t < kTok; ++t)
-      if (t < nt) inv[t] = row_inv_rms(a.x + (size_t)(t0 + t) * a.K, a.K, la.eps);
-    if (blockIdx.x == 0 && la.normed_out) {
-      for (int t = 0; t < nt; ++t) {
-        const float* xr = a.x + (size_t)(t0 + t) * a.K;
-        const float it = t == 0 ? inv[0] : t == 1 ? inv[1] : t == 2 ? inv[2] : t == 3 ? inv[3] : t == 4 ? inv[4] : t == 5 ? inv[5] : t == 6 ? inv[6] : inv[7];
-        for (int j = threadIdx.x; j < a.K; j += 256) la.normed_out[(size_t)(t0 + t) * a.K + j] = xr[j] * it * la.norm_w[j];
+        for (int t = 0; t < TOK; ++t) acc[r][m][t] = 0.0f;
+    float x[TOK][32];
+    Pending pend[R][NM];
+    // raw activations of step k.  Unconditional loads from clamped addresses (a token past the batch reads
+    // the last live one, a lane past the end of the row its last block): a select here would need the data
+    // at once and stall the pipeline; lanes past the row are zeroed where the values are used.
+    auto issue_x = [&](int k) __attribute__((always_inline)) {
+      const int koff = min(lane_koff<QUANT, 1>(g, k), a.K - F::kBlockElems);
+#pragma unroll
+      for (int t = 0; t < TOK; ++t) lane_x_load<QUANT>(a.x + (size_t)(t0 + min(t, nt - 1)) * a.K, koff, g, x[t]);
+      issue_fence();
+    };
+    auto issue_w = [&](int k) __attribute__((always_inline)) {
+      const bool act = lane_koff<QUANT, 1>(g, k) < a.K;
+      // live bytes of this step: whole blocks up to the end of the row
+      const uint32_t nbytes = (uint32_t)(min(kStepElems, a.K - k * kStepElems) / F::kBlockElems) * F::kBlockBytes;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const size_t off = (size_t)(row0 + r) * row_bytes + (size_t)k * F::kChunkBytes;
+        if constexpr (STAGED) {
+          stage_load<QUANT>(a.w0 + off, nbytes, pend[r][0]);
+          if constexpr (NM == 2) stage_load<QUANT>(a.w1 + off, nbytes, pend[r][NM - 1]);
+        } else {
+          load_raw<QUANT>(a.w0 + off, act, g, pend[r][0]);
+          if constexpr (NM == 2) load_raw<QUANT>(a.w1 + off, act, g, pend[r][NM - 1]);
+        }
       }
-    }
-  }
-  float acc[R][NM][kTok];
+      issue_fence();
+    };
+    issue_x(0);
+    issue_w(0);
+#pragma unroll 1
+    for (int k = 0; k < steps; ++k) {
+      const bool act = lane_koff<QUANT, 1>(g, k) < a.K;
+      float xl[TOK][32], xs[TOK][4];
 #pragma unroll
-  for (int r = 0; r < R; ++r)
+      for (int t = 0; t < TOK; ++t) {
 #pragma unroll
-    for (int m = 0; m < NM; ++m)
-#pragma unroll
-      for (int t = 0; t < kTok; ++t) acc[r][m][t] = 0.0f;
-  for (int k = 0; k < steps; ++k) {
-    const int koff = lane_koff<QUANT, 1>(g, k);
-    const bool act = koff < a.K;
-    load_step(k, raw);
-#pragma unroll
-    for (int c = 0; c < kTok / 2; ++c) {
-      if (2 * c >= nt) break;
-      if (2 * c + 1 < nt) {
-        float x[2][32], xs[2][4];
-        load_x<QUANT, XMODE>(a.x + (size_t)(t0 + 2 * c) * a.K, koff, act, g, x[0], xs[0], XNorm{inv[2 * c], la.norm_w});
-        load_x<QUANT, XMODE>(a.x + (size_t)(t0 + 2 * c + 1) * a.K, koff, act, g, x[1], xs[1], XNorm{inv[2 * c + 1], la.norm_w});
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-          for (int m = 0; m < NM; ++m) {
-            float tt[2] = {acc[r][m][2 * c], acc[r][m][2 * c + 1]};
-            accum<QUANT, 2>(raw[r][m], g, x, xs, tt);
-            acc[r][m][2 * c] = tt[0];
-            acc[r][m][2 * c + 1] = tt[1];
-          }
-      } else {
-        float x[1][32], xs[1][4];
-        load_x<QUANT, XMODE>(a.x + (size_t)(t0 + 2 * c) * a.K, koff, act, g, x[0], xs[0], XNorm{inv[2 * c], la.norm_w});
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-          for (int m = 0; m < NM; ++m) {
-            float tt[1] = {acc[r][m][2 * c]};
-            accum<QUANT, 1>(raw[r][m], g, x, xs, tt);
-            acc[r][m][2 * c] = tt[0];
-          }
+        for (int i = 0; i < 32; ++i) xl[t][i] = act ? x[t][i] : 0.0f;
+        lane_x_offsets<QUANT>(xl[t], xs[t]);
       }
+      Raw raw[R][NM];
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+          if constexpr (STAGED) stage_pick<QUANT>(pend[r][m], s_slots + (size_t)((wave * R + r) * NM + m) * kSlot, act, g, raw[r][m]);
+          else raw[r][m] = pend[r][m];
+        }
+      if (k + 1 < steps) issue_w(k + 1);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < NM; ++m) accum<QUANT, TOK>(raw[r][m], g, xl, xs, acc[r][m]);
+      if (k + 1 < steps) issue_x(k + 1);
     }
-  }
 #pragma unroll
-  for (int t = 0; t < kTok; ++t) {
-    if (t >= nt) break;
+    for (int t = 0; t < TOK; ++t) {
+      if (t >= nt) break;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      float tot[NM];
+      for (int r = 0; r < R; ++r) {
+        float tot[NM];
 #pragma unroll
-      for (int m = 0; m < NM; ++m) tot[m] = group_sum<64>(acc[r][m][t]);
-      if (g.lane == 0) {
-        const size_t i = (size_t)(t0 + t) * a.n_rows + row0 + r;
-        const float v = NM == 2 ? silu_f(tot[0]) * tot[NM - 1] : 1.0f * tot[0];
-        a.out[i] = v;
-        if constexpr (RESID) la.l_out[i] = v + la.residual[i];
+        for (int m = 0; m < NM; ++m) tot[m] = group_sum<64>(acc[r][m][t]);
+        if (g.lane == 0) {
+          const size_t i = (size_t)(t0 + t) * a.n_rows + row0 + r;
+          const float v = NM == 2 ? silu_f(tot[0]) * tot[NM - 1] : 1.0f * tot[0];
+          a.out[i] = v;
+          if constexpr (RESID) la.l_out[i] = v + la.residual[i];
+        }
       }
     }
   }

@@ -122,12 +122,16 @@ __device__ __forceinline__ float rms_finish(float lane_sum, int width, float eps
   return 1.0f / sqrtf(ss / (float)width + eps);
 }
 
+// Three chunks are requested together (a chunk past the end of the row loads nothing and folds zeros,
+// which leave the sum as it is), then folded in chunk order.
 __device__ __forceinline__ float row_inv_rms(const float* __restrict__ x, int width, float eps) {
   float s = 0.0f;
-  for (int c = 0; c < width; c += 2048) {
-    RmsRaw r;
-    rms_load(x, c, width, r);
-    s = rms_fold(r, s);
+  for (int c = 0; c < width; c += 3 * 2048) {
+    RmsRaw r[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) rms_load(x, c + 2048 * i, width, r[i]);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) s = rms_fold(r[i], s);
   }
   return rms_finish(s, width, eps);
 }

@@ -27,8 +27,30 @@ __global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__
                                                         float* __restrict__ out, int width, float eps) {
   const float* xr = x + (size_t)blockIdx.x * width;
   float* o = out + (size_t)blockIdx.x * width;
+  // width is a multiple of 4; the first eight float4 columns of every thread (rows up to 8192 wide) are
+  // requested together with the row's RMS chunks
+  const int n4 = width / 4;
+  const float4* x4 = reinterpret_cast<const float4*>(xr);
+  const float4* w4 = reinterpret_cast<const float4*>(w);
+  float4* o4 = reinterpret_cast<float4*>(o);
+  float4 xv[8], wv[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int j = min((int)threadIdx.x + 256 * i, n4 - 1);
+    xv[i] = x4[j];
+    wv[i] = w4[j];
+  }
   const float inv = row_inv_rms(xr, width, eps);  // each wavefront computes the same scale
-  for (int j = threadIdx.x; j < width; j += 256) o[j] = xr[j] * inv * w[j];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int j = threadIdx.x + 256 * i;
+    if (j < n4)
+      o4[j] = make_float4(xv[i].x * inv * wv[i].x, xv[i].y * inv * wv[i].y, xv[i].z * inv * wv[i].z, xv[i].w * inv * wv[i].w);
+  }
+  for (int j = threadIdx.x + 2048; j < n4; j += 256) {
+    const float4 a = x4[j], b = w4[j];
+    o4[j] = make_float4(a.x * inv * b.x, a.y * inv * b.y, a.z * inv * b.z, a.w * inv * b.w);
+  }
 }
 
 __global__ void __launch_bounds__(256) k_route(const float* __restrict__ logits, const int* __restrict__ valid_tokens,
