@@ -1,6 +1,6 @@
-// The decode-width MoE block (max_tokens <= 4) as three launches with no intermediate passes.
+// The decode-width MoE block (max_tokens <= 16) as three launches with no intermediate passes.
 //
-// At one to four tokens the block moves ~60 MB and every dependent memory access costs 1-2 us, so what
+// At a few tokens the block moves ~20 MB per token and every dependent memory access costs 1-2 us, so what
 // decides the time is the number of dependent round trips and launch boundaries on the critical path, not
 // bytes.  The eight steps of the block (norm, router, bias, route, gate/up, down, shared expert, combine)
 // are regrouped so that each launch issues everything it needs in one or two rounds of loads:
@@ -35,6 +35,7 @@ namespace xabe { static __device__ long long g_route_trace[4096 * 8]; }
 
 namespace xabe {
 
+constexpr size_t kDecodeBlockMaxTokens = 16;  // widest batch served by the three launches (the dispatch-table regime is faster from ~24 tokens)
 constexpr int kMaxTopK = 8;       // contributions held in registers by k_decode_down
 constexpr int kMaxInter = 512;    // intermediate width staged in LDS by k_decode_down
 
@@ -425,7 +426,7 @@ static bool launch_router(int router_quant, const Launch& l) {
 
 bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, const xabe_moe_layer_weights* w) {
   const xabe_moe_geometry& g = k->g;
-  if (g.max_tokens > kFlatMaxTokens || k->force_community || b->scope != XABE_SCOPE_ROUTED) return false;
+  if (g.max_tokens > kDecodeBlockMaxTokens || k->force_community || b->scope != XABE_SCOPE_ROUTED) return false;
   if (!((g.hidden == 2048 && g.intermediate == 512) || (g.hidden == 512 && g.intermediate == 256))) return false;
   if (g.experts_per_token > (size_t)kMaxTopK || g.num_experts > kRouteMaxExperts || g.num_experts % 4 != 0) return false;
   auto ok = [](int q) { return q == XABE_QUANT_Q6K || q == XABE_QUANT_Q8_0; };

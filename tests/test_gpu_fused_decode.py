@@ -1,5 +1,6 @@
-"""The decode-width block (max_tokens <= 4) regrouped into three launches against the same block with one
-launch per step: every observable tensor bit for bit, over repeated calls, with fewer live tokens than
+"""The decode-width block (max_tokens <= 16) regrouped into three launches against the same block with one
+launch per step (flat per-pair kernels up to 4 tokens, the dispatch-table regime above): every observable
+tensor bit for bit, over repeated calls, with fewer live tokens than
 the buffer holds, with and without a logit bias, and for each format pairing.  The per-step launches are
 the ones the oracle comparisons of test_gpu_decode.py cover; test_block_matches_oracle runs the regrouped
 block against the oracle directly."""
@@ -53,7 +54,8 @@ def _compare(X, oracle, g, tokens_seq, seed, router_q8=True, bias=False, expert_
         _same_bits(_observe(one, g, f1, l1, tokens), _observe(many, g, f2, l2, tokens), f"call {i} tokens {tokens}")
 
 
-@pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (2, (2, 1, 2)), (3, (3, 1, 2, 3)), (4, (4, 3, 0, 4, 1))])
+@pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (2, (2, 1, 2)), (3, (3, 1, 2, 3)), (4, (4, 3, 0, 4, 1)),
+                                                   (5, (5, 2, 5)), (8, (8, 1, 7)), (16, (16, 9, 0, 16))])
 @pytest.mark.parametrize("router_q8", [True, False])
 def test_small_geometry(oracle, X, max_tokens, tokens_seq, router_q8):
     g = X.MoeGeometry(8, 2, 512, 256, 32, max_tokens)
@@ -66,7 +68,7 @@ def test_small_geometry_format_pairings(oracle, X, eq, sq):
     _compare(X, oracle, g, (3, 2), seed=4200, expert_quant=getattr(X.ExpertQuant, eq), shared_quant=getattr(X.ExpertQuant, sq))
 
 
-@pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (3, (3, 3, 2)), (4, (4, 1, 4))])
+@pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (3, (3, 3, 2)), (4, (4, 1, 4)), (7, (7, 5)), (16, (16, 11))])
 def test_model_geometry(oracle, X, max_tokens, tokens_seq):
     g = X.MoeGeometry.qwen3_6(X.moe_block_size(max_tokens), max_tokens)
     _compare(X, oracle, g, tokens_seq, seed=4300 + max_tokens, bias=(max_tokens == 3))
