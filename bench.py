@@ -42,10 +42,15 @@ def main() -> int:
                          "traffic against which hardware byte counters of the same run are scaled")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--workload", default="decode_b3", choices=["decode_b3"] + sorted(OTHER_WORKLOADS),
+                    help="decode_b3 is the headline (everything above applies to it); the others are BASELINE's "
+                         "remaining configurations, timed whole-block with HIP events, for profiles and comparison")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         return 2
+    if args.workload != "decode_b3":
+        return other_workload(args)
 
     import numpy as np
     import torch
@@ -214,6 +219,86 @@ def main() -> int:
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(layers[0], g, x, T, args.cpu_seconds)
     print(json.dumps(out))
+    return 0
+
+
+MFMA_PEAK_TFLOPS = 2500.0
+# name -> (kind, tokens, layers rotated): the MoE block at other widths and the dense sibling
+OTHER_WORKLOADS = {"decode_b32": ("moe", 32, 16), "prefill_512": ("moe", 512, 4), "prefill_8192": ("moe", 8192, 2),
+                   "dense_b1": ("dense", 1, 4), "dense_b8": ("dense", 8, 4)}
+
+
+def other_workload(args) -> int:
+    """One of BASELINE's other configurations: the whole block, eager launches, HIP events on the launch
+    stream over rotated layers.  One JSON line in the headline's format; the roofline is the block's own
+    (algorithmic bytes or flops of a pass over its duration), not one kernel's."""
+    import numpy as np
+    import torch
+
+    import llmxabe_amd as X
+
+    torch.cuda.set_device(0)
+    kind, T, L = OTHER_WORKLOADS[args.workload]
+    if kind == "moe":
+        g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
+        layers = [make_layer_device_only(X, g, seed=10_000 + 100 * l) for l in range(L)]
+        blk = X.MoeBlock(g)
+        blk.publish_tokens(T)
+        width = 2048
+    else:
+        H, I = 5120, 17408
+        q = X.ExpertQuant.Q6K
+        layers = []
+        for l in range(L):
+            t = [X.QuantTensor(X.synth_quant(q, 41 + 10 * l + j, H * I, 0.02), q) for j in range(3)]
+            layers.append(X.DenseFfnLayerWeights(1.0 + X.synth_normal_f32(44 + 10 * l, H, 0.1), t[0], t[1], t[2]))
+        blk = X.DenseFfnBlock(H, I, T)
+        width = H
+    x = X.synth_normal_f32(99, T * width, 1.0).view(T, width)
+    ffn_out, l_out = torch.zeros_like(x), torch.zeros_like(x)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    reps_w = max(1, min(args.warmup, 64) // L)
+    reps = max(1, min(args.steps, 64 if T >= 512 else 320) // L)
+    with torch.cuda.stream(stream):
+        for _ in range(reps_w):
+            for i in range(L):
+                blk.forward(layers[i], x, T, ffn_out, l_out)
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            for i in range(L):
+                blk.forward(layers[i], x, T, ffn_out, l_out)
+        e1.record(stream)
+        e1.synchronize()
+    steps = reps * L
+    ms = e0.elapsed_time(e1) / steps
+    if kind == "moe":
+        ids = blk.buffers().topk_ids().cpu().numpy().reshape(T, 8)
+        distinct = len(np.unique(ids))
+        byts = distinct * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES + 16384 + T * 2048 * 4 * 3
+        flops = T * 57671680
+        cfg = {"workload": "moe_block_" + args.workload, "tokens": T, "num_experts": 256, "top_k": 8, "hidden": 2048,
+               "intermediate": 512, "expert_quant": "Q6_K", "shared_and_router_quant": "Q8_0", "layers_rotated": L,
+               "launch": "eager", "distinct_experts": distinct}
+    else:
+        byts = 3 * 5120 * 17408 // 256 * 210
+        flops = T * 3 * 2 * 5120 * 17408
+        cfg = {"workload": "dense_ffn_" + args.workload, "tokens": T, "hidden": 5120, "intermediate": 17408,
+               "quant": "Q6_K", "layers_rotated": L, "launch": "eager"}
+    gbps, tflops = byts / (ms * 1e-3) / 1e9, flops / (ms * 1e-3) / 1e12
+    mfma_bound = args.workload == "prefill_8192"
+    roof = ({"kernel": "whole block", "bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+             "frac": tflops / MFMA_PEAK_TFLOPS, "traffic": None} if mfma_bound else
+            {"kernel": "whole block", "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": gbps / HBM_PEAK_GBPS, "traffic": None})
+    print(json.dumps({
+        "metric": "MoE-block tokens/s at 1 GPU; decode HBM GB/s %peak; prefill MFMA util %", "value": T / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": reps_w * L, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if kind == "moe" and T >= 64 else "f32",
+        "data": "synthetic", "config": cfg, "roofline": roof, "algorithmic_bytes_per_step": byts, "flops_per_step": flops,
+        "cpu_baseline": None}))
     return 0
 
 

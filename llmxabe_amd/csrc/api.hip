@@ -828,7 +828,11 @@ int xabe_rms_norm(void* stream, const float* x, size_t x_len, const float* weigh
   if (width % 4 != 0) return set_error(XABE_ERR_INVALID_ARGUMENT, "rms_norm: width %zu is not a multiple of 4", width);
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out)) % 16 != 0)
     return set_error(XABE_ERR_INVALID_ARGUMENT, "rms_norm: x, weight and out must be 16-byte aligned");
-  hipLaunchKernelGGL(k_rms_norm_rows, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), x, weight, out, (int)width, eps);
+  if (width <= 2048 && rows >= 64)  // (a handful of rows: one workgroup per row finishes sooner)
+    hipLaunchKernelGGL(k_rms_norm_short_rows, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, as_stream(stream), x, weight, out,
+                       (int)rows, (int)width, eps);
+  else
+    hipLaunchKernelGGL(k_rms_norm_rows, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), x, weight, out, (int)width, eps);
   XABE_HIP_TRY(hipGetLastError());
   return XABE_OK;
 }

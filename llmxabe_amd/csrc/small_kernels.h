@@ -27,8 +27,8 @@ __global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__
                                                         float* __restrict__ out, int width, float eps) {
   const float* xr = x + (size_t)blockIdx.x * width;
   float* o = out + (size_t)blockIdx.x * width;
-  // width is a multiple of 4; the first eight float4 columns of every thread (rows up to 8192 wide) are
-  // requested together with the row's RMS chunks
+  // width is a multiple of 4; up to eight float4 columns per thread (rows up to 8192 wide) are requested
+  // together with the row's RMS chunks.  The guards are uniform, so the loads stay in flight together.
   const int n4 = width / 4;
   const float4* x4 = reinterpret_cast<const float4*>(xr);
   const float4* w4 = reinterpret_cast<const float4*>(w);
@@ -36,9 +36,11 @@ __global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__
   float4 xv[8], wv[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int j = min((int)threadIdx.x + 256 * i, n4 - 1);
-    xv[i] = x4[j];
-    wv[i] = w4[j];
+    if (256 * i < n4) {
+      const int j = min((int)threadIdx.x + 256 * i, n4 - 1);
+      xv[i] = x4[j];
+      wv[i] = w4[j];
+    }
   }
   const float inv = row_inv_rms(xr, width, eps);  // each wavefront computes the same scale
 #pragma unroll
@@ -51,6 +53,25 @@ __global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__
     const float4 a = x4[j], b = w4[j];
     o4[j] = make_float4(a.x * inv * b.x, a.y * inv * b.y, a.z * inv * b.z, a.w * inv * b.w);
   }
+}
+
+// Rows of at most 2048 elements: one wavefront per row, four rows per workgroup.  The lane's 32 elements
+// are the ones rms_fold takes from it, so the row is read once and normalised out of the same registers.
+__global__ void __launch_bounds__(256) k_rms_norm_short_rows(const float* __restrict__ x, const float* __restrict__ w,
+                                                              float* __restrict__ out, int rows, int width, float eps) {
+  const int row = blockIdx.x * 4 + (int)(threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* xr = x + (size_t)row * width;
+  RmsRaw r, nw;
+  rms_load(xr, 0, width, r);
+  rms_load(w, 0, width, nw);
+  const float inv = rms_finish(rms_fold(r, 0.0f), width, eps);
+  const int base = (int)__lane_id() * 32;
+  float4* o4 = reinterpret_cast<float4*>(out + (size_t)row * width + base);
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    if (base + 4 * i < width)
+      o4[i] = make_float4(r.q[i].x * inv * nw.q[i].x, r.q[i].y * inv * nw.q[i].y, r.q[i].z * inv * nw.q[i].z, r.q[i].w * inv * nw.q[i].w);
 }
 
 __global__ void __launch_bounds__(256) k_route(const float* __restrict__ logits, const int* __restrict__ valid_tokens,
