@@ -169,34 +169,28 @@ bool launch_long_rows(const xabe_moe_kernels* k, int quant, int nm, const LongRo
   // the coalesced loader reads whole 16-byte pieces: the tensors must start and end on 16-byte boundaries
   const size_t row_bytes = (size_t)a.K / xabe_expert_quant_block_elements(quant) * xabe_expert_quant_block_bytes(quant);
   auto on16 = [&](const uint8_t* w) { return !w || (reinterpret_cast<uintptr_t>(w) % 16 == 0 && ((size_t)a.n_rows * row_bytes) % 16 == 0); };
-  const bool staged = on16(a.w0) && on16(a.w1);
-#define XABE_LONG4(Q, ST, TOK, R)                                                                                    \
-  do {                                                                                                                \
-    if (nm == 2) hipLaunchKernelGGL((k_shared_long_rows<Q, 2, R, TOK, false, ST>), grid, block, 0, s, la);            \
-    else if (resid) hipLaunchKernelGGL((k_shared_long_rows<Q, 1, R, TOK, true, ST>), grid, block, 0, s, la);          \
-    else hipLaunchKernelGGL((k_shared_long_rows<Q, 1, R, TOK, false, ST>), grid, block, 0, s, la);                \
+  if (!(on16(a.w0) && on16(a.w1))) return false;
+#define XABE_LONG4(Q, TOK, R)                                                                                    \
+  do {                                                                                                            \
+    if (nm == 2) hipLaunchKernelGGL((k_shared_long_rows<Q, 2, R, TOK, false>), grid, block, 0, s, la);            \
+    else if (resid) hipLaunchKernelGGL((k_shared_long_rows<Q, 1, R, TOK, true>), grid, block, 0, s, la);          \
+    else hipLaunchKernelGGL((k_shared_long_rows<Q, 1, R, TOK, false>), grid, block, 0, s, la);                    \
   } while (0)
-#define XABE_LONG3(Q, ST, TOK)                              \
-  do {                                                      \
-    if (nm == 2) XABE_LONG4(Q, ST, TOK, 2);                 \
-    else XABE_LONG4(Q, ST, TOK, 4);                         \
+#define XABE_LONG3(Q, TOK)                              \
+  do {                                                  \
+    if (nm == 2) XABE_LONG4(Q, TOK, 2);                 \
+    else XABE_LONG4(Q, TOK, 4);                         \
   } while (0)
-#define XABE_LONG2(Q, ST)                 \
-  do {                                    \
-    if (tok == 1) XABE_LONG3(Q, ST, 1);   \
-    else XABE_LONG3(Q, ST, 2);            \
-  } while (0)
-#define XABE_LONG(Q)                      \
-  do {                                    \
-    if (staged) XABE_LONG2(Q, true);      \
-    else XABE_LONG2(Q, false);            \
+#define XABE_LONG(Q)                  \
+  do {                                \
+    if (tok == 1) XABE_LONG3(Q, 1);   \
+    else XABE_LONG3(Q, 2);            \
   } while (0)
   if (quant == XABE_QUANT_Q6K) XABE_LONG(kQ6K);
   else XABE_LONG(kQ8_0);
 #undef XABE_LONG4
 #undef XABE_LONG3
 #undef XABE_LONG
-#undef XABE_LONG2
   return true;
 }
 

@@ -607,7 +607,8 @@ __device__ __forceinline__ void issue_fence() {
 // the weights (later passes find most of them in the memory-side cache); 64 or 256 threads.
 //   Software pipeline: the next step's weights are requested before this step's accumulation and its
 //   activations right after it, into the registers the accumulation has just released.
-//   STAGED: weights through the coalesced loader (stage_load / stage_pick); otherwise per-lane field loads.
+//   Weights come through the coalesced loader (stage_load / stage_pick): the host takes this kernel only for
+//   tensors that start and end on 16-byte boundaries.
 //   RESID:  also write l_out = out + residual (the dense block's last step).
 struct LongRowArgs {
   ExpertArgs m;
@@ -615,13 +616,12 @@ struct LongRowArgs {
   float* l_out;           // RESID
 };
 
-template <int QUANT, int NM, int R, int TOK, bool RESID, bool STAGED>
+template <int QUANT, int NM, int R, int TOK, bool RESID>
 __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
   using F = Fmt<QUANT>;
   using Raw = typename F::Raw;
-  using Pending = typename std::conditional<STAGED, Staged<QUANT>, Raw>::type;
   constexpr int kSlot = StageFmt<QUANT>::kSlotBytes;
-  __shared__ __attribute__((aligned(16))) uint8_t s_slots[STAGED ? kWavesPerWg * R * NM * kSlot : 16];
+  __shared__ __attribute__((aligned(16))) uint8_t s_slots[kWavesPerWg * R * NM * kSlot];
   const ExpertArgs& a = la.m;
   const int valid = *a.valid_tokens;
   const int t0 = blockIdx.y * TOK;
@@ -643,7 +643,7 @@ __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
 #pragma unroll
         for (int t = 0; t < TOK; ++t) acc[r][m][t] = 0.0f;
     float x[TOK][32];
-    Pending pend[R][NM];
+    Staged<QUANT> pend[R][NM];
     // raw activations of step k.  Unconditional loads from clamped addresses (a token past the batch reads
     // the last live one, a lane past the end of the row its last block): a select here would need the data
     // at once and stall the pipeline; lanes past the row are zeroed where the values are used.
@@ -654,19 +654,13 @@ __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
       issue_fence();
     };
     auto issue_w = [&](int k) __attribute__((always_inline)) {
-      const bool act = lane_koff<QUANT, 1>(g, k) < a.K;
       // live bytes of this step: whole blocks up to the end of the row
       const uint32_t nbytes = (uint32_t)(min(kStepElems, a.K - k * kStepElems) / F::kBlockElems) * F::kBlockBytes;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const size_t off = (size_t)(row0 + r) * row_bytes + (size_t)k * F::kChunkBytes;
-        if constexpr (STAGED) {
-          stage_load<QUANT>(a.w0 + off, nbytes, pend[r][0]);
-          if constexpr (NM == 2) stage_load<QUANT>(a.w1 + off, nbytes, pend[r][NM - 1]);
-        } else {
-          load_raw<QUANT>(a.w0 + off, act, g, pend[r][0]);
-          if constexpr (NM == 2) load_raw<QUANT>(a.w1 + off, act, g, pend[r][NM - 1]);
-        }
+        stage_load<QUANT>(a.w0 + off, nbytes, pend[r][0]);
+        if constexpr (NM == 2) stage_load<QUANT>(a.w1 + off, nbytes, pend[r][NM - 1]);
       }
       issue_fence();
     };
@@ -686,10 +680,8 @@ __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
 #pragma unroll
       for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int m = 0; m < NM; ++m) {
-          if constexpr (STAGED) stage_pick<QUANT>(pend[r][m], s_slots + (size_t)((wave * R + r) * NM + m) * kSlot, act, g, raw[r][m]);
-          else raw[r][m] = pend[r][m];
-        }
+        for (int m = 0; m < NM; ++m)
+          stage_pick<QUANT>(pend[r][m], s_slots + (size_t)((wave * R + r) * NM + m) * kSlot, act, g, raw[r][m]);
       if (k + 1 < steps) issue_w(k + 1);
 #pragma unroll
       for (int r = 0; r < R; ++r)
