@@ -113,13 +113,14 @@ struct WRaw {
   typename std::conditional<QUANT == kQ6K, Q6Raw, Q8Raw>::type u[2];
 };
 
-// Global loads of one contraction step into registers: eight 16-byte activation chunks and the
-// raw blocks of this thread's two weight-row units.
-template <int QUANT>
-__device__ __forceinline__ void load_step(int ks, const _Float16* const (&arow_ptr)[8], const uint8_t* const (&wrow)[2],
-                                          int du, u32x4 (&areg)[8], WRaw<QUANT>& wreg) {
+// Global loads of one contraction step into registers: eight 16-byte activation chunks ...
+__device__ __forceinline__ void load_step_a(int ks, const _Float16* const (&arow_ptr)[8], u32x4 (&areg)[8]) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const u32x4*>(arow_ptr[i] + (size_t)ks * kBK);
+}
+// ... and the raw blocks of this thread's two weight-row units.
+template <int QUANT>
+__device__ __forceinline__ void load_step_w(int ks, const uint8_t* const (&wrow)[2], int du, WRaw<QUANT>& wreg) {
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     if constexpr (QUANT == kQ6K) {
@@ -218,10 +219,18 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
+    // In flight: the next step's activation chunks (one matrix phase ahead: they come from L2) and the raw
+    // weight bytes of the next two steps (the HBM-cold ones), in w[ks & 1].  The contraction has an even
+    // number of steps (whole superblocks), so the step pairs are unrolled and no register is copied.
+    // (The down launch, NM = 1, has no registers to spare for the second step and keeps one in flight.)
+    constexpr int kWDepth = NM == 2 ? 2 : 1;
     u32x4 areg[8];
-    WRaw<QUANT> wreg;
-    load_step<QUANT>(0, arow_ptr, wrow, du, areg, wreg);
-    for (int ks = 0; ks < nks; ++ks) {
+    WRaw<QUANT> w[kWDepth];
+    load_step_w<QUANT>(0, wrow, du, w[0]);
+    load_step_a(0, arow_ptr, areg);
+    if constexpr (kWDepth == 2) load_step_w<QUANT>(1, wrow, du, w[kWDepth - 1]);
+    auto step = [&](auto p_c, int ks) __attribute__((always_inline)) {
+      constexpr int P = decltype(p_c)::value % kWDepth;
       __syncthreads();  // everyone has finished reading the previous step's tiles
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -231,11 +240,12 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int rb = rb0 + 64 * i;
-        if constexpr (QUANT == kQ6K) q6_unit_to_lds(wreg.u[i], du, &sB[rb * kLd]);
-        else q8_unit_to_lds(wreg.u[i], &sB[rb * kLd + du * 32]);
+        if constexpr (QUANT == kQ6K) q6_unit_to_lds(w[P].u[i], du, &sB[rb * kLd]);
+        else q8_unit_to_lds(w[P].u[i], &sB[rb * kLd + du * 32]);
       }
       __syncthreads();
-      if (ks + 1 < nks) load_step<QUANT>(ks + 1, arow_ptr, wrow, du, areg, wreg);  // in flight while the matrix cores work
+      if (ks + 1 < nks) load_step_a(ks + 1, arow_ptr, areg);  // in flight while the matrix cores work
+      if (ks + kWDepth < nks) load_step_w<QUANT>(ks + kWDepth, wrow, du, w[P]);
       const _Float16* pa = &sA[(wm * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
       const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
 #pragma unroll
@@ -249,6 +259,15 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
         acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, acc[1][0], 0, 0, 0);
         acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc[1][1], 0, 0, 0);
       }
+    };
+    if constexpr (kWDepth == 2) {
+      for (int ks = 0; ks < nks; ks += 2) {
+        step(std::integral_constant<int, 0>{}, ks);
+        step(std::integral_constant<int, 1>{}, ks + 1);
+      }
+    } else {
+#pragma unroll 1
+      for (int ks = 0; ks < nks; ++ks) step(std::integral_constant<int, 0>{}, ks);
     }
 
     // epilogue.  acc[mi][ni][v]: tile row (v/4)*8 + (lane/32)*4 + v%4, tile column lane%32
