@@ -70,7 +70,8 @@ struct DecodeArgs {
   float* routed;
   float* ffn_out;
   float* l_out;
-  size_t expert_bytes;  // bytes of one expert's matrix (gate, up and down are the same size)
+  size_t expert_bytes;  // bytes of one expert's gate (= up) matrix
+  size_t down_bytes;    // bytes of one expert's down matrix (its format may differ)
   float eps;
   int H, I, E, top_k, max_tokens;
   int tiles_r, tiles_s, tiles_g, tiles_d;  // row tiles: router, shared gate/up (launch A), gate/up (B), down (C)
@@ -345,7 +346,7 @@ __global__ void __launch_bounds__(256) k_decode_down(DecodeArgs a) {
     const int e = min(max(__builtin_amdgcn_readlane(my_e, k), 0), a.E - 1);
     // k >= top_k reads expert 0's rows and never uses them: an unconditional load keeps all of round two
     // in one basic block, so every load is issued before the first wait
-    load_raw<RQ>(a.down + (size_t)e * a.expert_bytes + (size_t)row0 * rb_r, true, gr, rr[k]);
+    load_raw<RQ>(a.down + (size_t)e * a.down_bytes + (size_t)row0 * rb_r, true, gr, rr[k]);
   }
   // the activation rows arrived before the weights (loads return in order); publish them to LDS
 #pragma unroll
@@ -397,30 +398,40 @@ struct Launch {
   unsigned launches;  // bit i: issue launch i (A, B, C); all three outside measurements
 };
 
-template <int RQ, int SQ, int RF, int RPSH, int DEPTH, int RPSI>
-static void launch_all(const Launch& l) {
-  if (l.launches & 1u) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);
-  if (l.launches & 2u) hipLaunchKernelGGL((k_decode_up<RQ, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
-  if (l.launches & 4u) hipLaunchKernelGGL((k_decode_down<RQ, SQ, RPSI>), dim3(l.grid_c), dim3(256), 0, l.s, l.a);
+// Each launch is chosen by the formats it reads: A by the shared gate/up and router formats, B by the routed
+// gate/up format, C by the routed and shared down formats (the shipped layers mix them: gate/up Q6_K with
+// down Q8_0).
+template <int RPSH, int DEPTH, int RPSI>
+static bool launch_all(const Launch& l, int gq, int dq, int sgq, int sdq, int router_quant) {
+  const bool g6 = gq == XABE_QUANT_Q6K, d6 = dq == XABE_QUANT_Q6K, sg6 = sgq == XABE_QUANT_Q6K, sd6 = sdq == XABE_QUANT_Q6K;
+  const bool rf32 = router_quant < 0;
+  if (!rf32 && router_quant != XABE_QUANT_Q8_0) return false;
+  if (l.launches & 1u) {
+#define XABE_A(SQ, RF) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH>), dim3(l.grid_a), dim3(256), 0, l.s, l.a)
+    if (sg6 && rf32) XABE_A(kQ6K, kF32);
+    else if (sg6) XABE_A(kQ6K, kQ8_0);
+    else if (rf32) XABE_A(kQ8_0, kF32);
+    else XABE_A(kQ8_0, kQ8_0);
+#undef XABE_A
+  }
+  if (l.launches & 2u) {
+    if (g6) hipLaunchKernelGGL((k_decode_up<kQ6K, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
+    else hipLaunchKernelGGL((k_decode_up<kQ8_0, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
+  }
+  if (l.launches & 4u) {
+#define XABE_C(RQ, SQ) hipLaunchKernelGGL((k_decode_down<RQ, SQ, RPSI>), dim3(l.grid_c), dim3(256), 0, l.s, l.a)
+    if (d6 && sd6) XABE_C(kQ6K, kQ6K);
+    else if (d6) XABE_C(kQ6K, kQ8_0);
+    else if (sd6) XABE_C(kQ8_0, kQ6K);
+    else XABE_C(kQ8_0, kQ8_0);
+#undef XABE_C
+  }
+  return true;
 }
 
-template <int RQ, int SQ, int RF>
-static bool launch_shape(const Launch& l) {
-  if (l.a.H == 2048 && l.a.I == 512) {
-    launch_all<RQ, SQ, RF, 1, 4, 4>(l);
-    return true;
-  }
-  if (l.a.H == 512 && l.a.I == 256) {
-    launch_all<RQ, SQ, RF, 4, 1, 8>(l);
-    return true;
-  }
-  return false;
-}
-
-template <int RQ, int SQ>
-static bool launch_router(int router_quant, const Launch& l) {
-  if (router_quant < 0) return launch_shape<RQ, SQ, kF32>(l);
-  if (router_quant == XABE_QUANT_Q8_0) return launch_shape<RQ, SQ, kQ8_0>(l);
+static bool launch_shape(const Launch& l, int gq, int dq, int sgq, int sdq, int router_quant) {
+  if (l.a.H == 2048 && l.a.I == 512) return launch_all<1, 4, 4>(l, gq, dq, sgq, sdq, router_quant);
+  if (l.a.H == 512 && l.a.I == 256) return launch_all<4, 1, 8>(l, gq, dq, sgq, sdq, router_quant);
   return false;
 }
 
@@ -430,9 +441,8 @@ bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b
   if (!((g.hidden == 2048 && g.intermediate == 512) || (g.hidden == 512 && g.intermediate == 256))) return false;
   if (g.experts_per_token > (size_t)kMaxTopK || g.num_experts > kRouteMaxExperts || g.num_experts % 4 != 0) return false;
   auto ok = [](int q) { return q == XABE_QUANT_Q6K || q == XABE_QUANT_Q8_0; };
-  if (!ok(w->gate_exps.quant) || w->gate_exps.quant != w->up_exps.quant || w->down_exps.quant != w->gate_exps.quant) return false;
-  if (!ok(w->shared_gate.quant) || w->shared_gate.quant != w->shared_up.quant || w->shared_down.quant != w->shared_gate.quant)
-    return false;
+  if (!ok(w->gate_exps.quant) || w->gate_exps.quant != w->up_exps.quant || !ok(w->down_exps.quant)) return false;
+  if (!ok(w->shared_gate.quant) || w->shared_gate.quant != w->shared_up.quant || !ok(w->shared_down.quant)) return false;
   if (!(w->router_quant < 0 || w->router_quant == XABE_QUANT_Q8_0)) return false;
   return true;
 }
@@ -466,8 +476,9 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
   a.routed = routed;
   a.ffn_out = ffn_out;
   a.l_out = l_out;
-  const int rq = w->gate_exps.quant, sq = w->shared_gate.quant;
+  const int rq = w->gate_exps.quant, dq = w->down_exps.quant;
   a.expert_bytes = g.intermediate * g.hidden / xabe_expert_quant_block_elements(rq) * xabe_expert_quant_block_bytes(rq);
+  a.down_bytes = g.intermediate * g.hidden / xabe_expert_quant_block_elements(dq) * xabe_expert_quant_block_bytes(dq);
   a.eps = eps;
   a.H = (int)g.hidden;
   a.I = (int)g.intermediate;
@@ -488,11 +499,7 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
   l.grid_a = (unsigned)(chunks * (a.tiles_r + a.tiles_s) + a.max_tokens);
   l.grid_b = (unsigned)(a.max_tokens * a.top_k * a.tiles_g);
   l.grid_c = (unsigned)(a.max_tokens * a.tiles_d);
-  bool ok;
-  if (rq == XABE_QUANT_Q6K && sq == XABE_QUANT_Q6K) ok = launch_router<kQ6K, kQ6K>(w->router_quant, l);
-  else if (rq == XABE_QUANT_Q6K && sq == XABE_QUANT_Q8_0) ok = launch_router<kQ6K, kQ8_0>(w->router_quant, l);
-  else if (rq == XABE_QUANT_Q8_0 && sq == XABE_QUANT_Q6K) ok = launch_router<kQ8_0, kQ6K>(w->router_quant, l);
-  else ok = launch_router<kQ8_0, kQ8_0>(w->router_quant, l);
+  const bool ok = launch_shape(l, w->gate_exps.quant, w->down_exps.quant, w->shared_gate.quant, w->shared_down.quant, w->router_quant);
   if (!ok) return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "decode block: no kernels for this shape or format");
   XABE_HIP_TRY(hipGetLastError());
   return XABE_OK;

@@ -164,14 +164,17 @@ def test_weight_stack_checks(oracle, X):
         k.grouped_forward_partial(so, d.gate_exps, d.up_exps, d.down_exps, x)
 
 
-@pytest.mark.parametrize("max_tokens,tokens,router_q8", [(1, 1, True), (3, 3, True), (3, 3, False), (4, 2, True),
-                                                         (32, 32, True), (48, 37, False)])
-def test_block_matches_oracle(oracle, X, max_tokens, tokens, router_q8):
+@pytest.mark.parametrize("max_tokens,tokens,router_q8,down_q8", [
+    (1, 1, True, False), (3, 3, True, False), (3, 3, False, False), (4, 2, True, False), (32, 32, True, False),
+    (48, 37, False, False),
+    # the shipped layers' layout: gate/up Q6_K, down Q8_0, f32 router
+    (3, 3, False, True), (12, 9, False, True), (32, 32, False, True)])
+def test_block_matches_oracle(oracle, X, max_tokens, tokens, router_q8, down_q8):
     """Whole block.  Routing contract: the ids are what route_token returns for the device's own logits
     (the reference's method, crates/xabe-engine/tests/moe_block.rs:1012-1016); logits vs the sequential
     gemv at reassociation tolerance; block outputs at DECODE_REL of peak."""
     g = X.MoeGeometry.qwen3_6(32, max_tokens)
-    layer = make_layer(oracle, g, seed=700, router_q8=router_q8)
+    layer = make_layer(oracle, g, seed=700, router_q8=router_q8, down_quant=X.ExpertQuant.Q8_0 if down_q8 else None)
     x = activations(15, max_tokens, 2048, tokens)
     blk = X.MoeBlock(g)
     ffn_out, l_out = run_block(blk, layer, x, tokens)

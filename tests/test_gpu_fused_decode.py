@@ -40,10 +40,12 @@ def _same_bits(a, b, what):
         assert np.array_equal(x, y), f"{what}: {key} differs"
 
 
-def _compare(X, oracle, g, tokens_seq, seed, router_q8=True, bias=False, expert_quant=None, shared_quant=None):
+def _compare(X, oracle, g, tokens_seq, seed, router_q8=True, bias=False, expert_quant=None, shared_quant=None,
+             down_quant=None, shared_down_quant=None):
     import torch
 
-    layer = make_layer(oracle, g, seed=seed, router_q8=router_q8, expert_quant=expert_quant, shared_quant=shared_quant)
+    layer = make_layer(oracle, g, seed=seed, router_q8=router_q8, expert_quant=expert_quant, shared_quant=shared_quant,
+                       down_quant=down_quant, shared_down_quant=shared_down_quant)
     one, many = X.MoeBlock(g), X.MoeBlock(g)
     many.set_fused_decode(False)
     lb = X.synth_normal_f32(seed + 77, g.num_experts, 1.0) if bias else None
@@ -66,6 +68,27 @@ def test_small_geometry(oracle, X, max_tokens, tokens_seq, router_q8):
 def test_small_geometry_format_pairings(oracle, X, eq, sq):
     g = X.MoeGeometry(16, 4, 512, 256, 32, 3)
     _compare(X, oracle, g, (3, 2), seed=4200, expert_quant=getattr(X.ExpertQuant, eq), shared_quant=getattr(X.ExpertQuant, sq))
+
+
+@pytest.mark.parametrize("eq,dq,sq,sdq", [("Q6K", "Q8_0", "Q8_0", "Q8_0"), ("Q8_0", "Q6K", "Q6K", "Q8_0"),
+                                         ("Q6K", "Q8_0", "Q8_0", "Q6K")])
+def test_small_geometry_mixed_formats(oracle, X, eq, dq, sq, sdq):
+    # down projections in another format than gate/up, as in the shipped layers (gate/up Q6_K, down Q8_0)
+    q = lambda n: getattr(X.ExpertQuant, n)
+    g = X.MoeGeometry(16, 4, 512, 256, 32, 3)
+    _compare(X, oracle, g, (3, 1), seed=4250, expert_quant=q(eq), shared_quant=q(sq), down_quant=q(dq), shared_down_quant=q(sdq))
+
+
+def test_model_geometry_shipped_layout(oracle, X):
+    # gate/up Q6_K, down Q8_0, shared expert Q8_0, f32 router
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(3), 3)
+    _compare(X, oracle, g, (3, 2), seed=4350, router_q8=False, down_quant=X.ExpertQuant.Q8_0)
+    # and the three launches really serve it: the single-launch hook refuses layouts they do not cover
+    layer = make_layer(oracle, g, seed=4350, router_q8=False, down_quant=X.ExpertQuant.Q8_0)
+    blk = X.MoeBlock(g)
+    x = activations(4360, 3, 2048, 3)
+    f, l = run_block(blk, layer, x, 3)
+    blk.forward_stage(layer.dev, x, f, l, 2)
 
 
 @pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (3, (3, 3, 2)), (4, (4, 1, 4)), (7, (7, 5)), (16, (16, 11))])
