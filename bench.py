@@ -190,20 +190,37 @@ def main() -> int:
                      for n, u, bts in zip(stage_names, stage_us, stage_bytes)],
     }
 
-    # ---- what this box can do, next to the nominal peaks: a plain device read and a plain fp16 GEMM,
-    # both library routines (nothing of this repository is in them)
+    # ---- what this box can do, next to the nominal peaks: a pure coalesced 16-byte-per-lane read of 2 GiB
+    # (eight times the 256 MB Infinity Cache) and a register-resident fp16 matrix-instruction loop, both
+    # kernels of this library's calibrate.hip; and, for comparison, two library routines
     with torch.cuda.stream(stream):
-        big = torch.ones(1 << 28, dtype=torch.int32, device="cuda")   # 1 GiB
-        dst = torch.empty_like(big)
-        dst.copy_(big)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        big = torch.ones(1 << 29, dtype=torch.int32, device="cuda")   # 2 GiB
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        X.calibrate_hbm_read(big, sink)
         e0.record(stream)
         for _ in range(5):
-            dst.copy_(big)
+            X.calibrate_hbm_read(big, sink)
         e1.record(stream)
         e1.synchronize()
-        read_gbps = 5 * 2 * big.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
-        del big, dst
+        read_gbps = 5 * big.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+        half = big[: 1 << 28]
+        dst = torch.empty_like(half)
+        dst.copy_(half)
+        e0.record(stream)
+        for _ in range(5):
+            dst.copy_(half)
+        e1.record(stream)
+        e1.synchronize()
+        copy_gbps = 5 * 2 * half.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+        del big, half, dst
+        mout = torch.zeros(512 * 1024, dtype=torch.float32, device="cuda")
+        X.calibrate_mfma_f16(mout, 2000)
+        e0.record(stream)
+        mflops = X.calibrate_mfma_f16(mout, 20000)
+        e1.record(stream)
+        e1.synchronize()
+        mfma_tflops = mflops / (e0.elapsed_time(e1) * 1e-3) / 1e12
         ma = torch.randn(8192, 8192, device="cuda", dtype=torch.float16)
         mb = torch.randn(8192, 8192, device="cuda", dtype=torch.float16)
         torch.matmul(ma, mb)
@@ -214,7 +231,9 @@ def main() -> int:
         e1.synchronize()
         gemm_tflops = 5 * 2 * 8192 ** 3 / (e0.elapsed_time(e1) * 1e-3) / 1e12
         del ma, mb
-    out["calibration"] = {"device_copy_gbps": read_gbps, "device_copy_what": "torch copy of 1 GiB, bytes read + written",
+    out["calibration"] = {"hbm_read_gbps": read_gbps, "hbm_read_what": "coalesced 16-byte-per-lane read of 2 GiB (xabe_calibrate_hbm_read)",
+                          "mfma_f16_tflops": mfma_tflops, "mfma_f16_what": "register-resident v_mfma_f32_32x32x16_f16 loop, two wavefronts per SIMD (xabe_calibrate_mfma_f16)",
+                          "device_copy_gbps": copy_gbps, "device_copy_what": "torch copy of 1 GiB, bytes read + written",
                           "fp16_gemm_tflops": gemm_tflops, "fp16_gemm_what": "torch.matmul 8192^3 fp16 (hipBLASLt)"}
 
     if not args.no_cpu:

@@ -271,6 +271,15 @@ const float* xabe_dense_ffn_block_normed(const xabe_dense_ffn_block* blk, size_t
 int xabe_synth_normal_f32(void* stream, uint64_t seed, size_t n, float sigma, float* out);
 int xabe_synth_quant(void* stream, int quant, uint64_t seed, size_t n_elements, float sigma, void* out, size_t out_len);
 
+/* ---- what the part reaches, measured as the reference measures its card (no counterpart among the
+ * reference's library calls; crates/xabe-cuda/src/bin/bench_dense_ffn.rs:88-111 does the read in its bench,
+ * docs/BENCHMARKS.md:1022-1024 the matrix-instruction loop).  One launch per call; the caller times it. ----
+ * xabe_calibrate_hbm_read: every 16-byte piece of `buffer` read once, coalesced.
+ * xabe_calibrate_mfma_f16: a register-resident loop of 32x32x16 fp16 matrix instructions on every SIMD;
+ *   `out` needs 512 floats per CU; `*flops` receives the floating-point operations of the launch. */
+int xabe_calibrate_hbm_read(void* stream, const void* buffer, size_t bytes, void* sink);
+int xabe_calibrate_mfma_f16(void* stream, float* out, size_t out_len, int iters, double* flops);
+
 #ifdef __cplusplus
 }
 #endif

@@ -109,6 +109,8 @@ _SIGNATURES = {
     "xabe_dense_ffn_block_disable_tensor_cores": (C.c_int, [vp]),
     "xabe_dense_ffn_block_normed": (vp, [vp, C.POINTER(sz)]),
     "xabe_synth_normal_f32": (C.c_int, [vp, C.c_uint64, sz, C.c_float, vp]),
+    "xabe_calibrate_hbm_read": (C.c_int, [vp, vp, sz, vp]),
+    "xabe_calibrate_mfma_f16": (C.c_int, [vp, vp, sz, C.c_int, C.POINTER(C.c_double)]),
     "xabe_synth_quant": (C.c_int, [vp, C.c_int, C.c_uint64, sz, C.c_float, vp, sz]),
 }
 

@@ -307,6 +307,18 @@ def synth_normal_f32(seed: int, n: int, sigma: float) -> torch.Tensor:
     return out
 
 
+def calibrate_hbm_read(buffer: torch.Tensor, sink: torch.Tensor) -> None:
+    """One launch that reads every 16-byte piece of `buffer` once, coalesced; the caller times it."""
+    check(_ffi.lib().xabe_calibrate_hbm_read(_stream(), _ptr(buffer), buffer.numel() * buffer.element_size(), _ptr(sink)))
+
+
+def calibrate_mfma_f16(out: torch.Tensor, iters: int) -> float:
+    """One launch of a register-resident fp16 matrix-instruction loop on every SIMD; returns its flop count."""
+    flops = C.c_double(0.0)
+    check(_ffi.lib().xabe_calibrate_mfma_f16(_stream(), _ptr(out), out.numel(), iters, C.byref(flops)))
+    return flops.value
+
+
 def synth_quant(quant: ExpertQuant, seed: int, n_elements: int, sigma: float) -> torch.Tensor:
     q = ExpertQuant(quant)
     nbytes = n_elements // q.block_elements() * q.block_bytes()
