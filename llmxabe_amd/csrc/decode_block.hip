@@ -22,6 +22,8 @@
 // bit-identical to it and to the wider regimes: the batch-invariance contract is unchanged.
 #include <string.h>
 
+#include <type_traits>
+
 #include "decode_kernels.h"
 #include "host_common.h"
 #ifdef XABE_TRACE_ITEMS
@@ -231,7 +233,7 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   using Raw = typename F::Raw;
   constexpr int G = 64 / RPS;
   extern __shared__ float s_route[];  // num_experts floats for the routing wavefront
-  __shared__ int s_expert;
+  __shared__ int s_expert, s_final;  // the candidate expert of this pair; the one routing settles on
   const int p = blockIdx.x / a.tiles_g, tile = blockIdx.x % a.tiles_g;
   const int t = p / a.top_k, k = p % a.top_k;
   // everything read before the live-token count is known is sized for max_tokens rows
@@ -252,45 +254,77 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   float x[1][32], xs[1][4];
   lane_x_load<RQ>(a.normed + (size_t)t * a.H, koff, g, x[0]);
   if (t >= valid) return;
+  // Routing in two halves (route_device.h).  The first orders the experts by logit: its k-th candidate is
+  // the pair's expert unless probabilities tie, and it is known ~2 us before the softmax is, so the four
+  // wavefronts request the candidate's rows right away.  The routing wavefront then finishes the softmax
+  // under its own loads' latency; in the rare pass where the probabilities reorder the candidates, the rows
+  // are streamed again for the expert the reference's rule selects.
+  const int n_cand = min(a.top_k + 1, a.E);
+  int cand_i = 0;
   if (routes) {
-    int sel_i;
-    float sel_w;
     XABE_ROUTE_TRACE(0);
-    if (few) route_compute<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, a.top_k, s_route, sel_i, sel_w);
-    else route_compute<kRouteMaxPerLane>(lg, a.E, a.top_k, s_route, sel_i, sel_w);
-    XABE_ROUTE_TRACE(5);
-    if (g.lane == k) s_expert = sel_i;
-    if (k == 0 && tile == 0 && g.lane < a.top_k) {
-      a.topk_ids[(size_t)t * a.top_k + g.lane] = sel_i;
-      a.topk_weights[(size_t)t * a.top_k + g.lane] = sel_w;
-    }
+    if (few) route_order<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, n_cand, cand_i);
+    else route_order<kRouteMaxPerLane>(lg, a.E, n_cand, cand_i);
+    if (g.lane == k) s_expert = cand_i;
   }
   lane_x_offsets<RQ>(x[0], xs[0]);
   __syncthreads();
   XABE_TRACE(1, 1);
-  const int e = s_expert;
   const size_t row_bytes = (size_t)(a.H / F::kBlockElems) * F::kBlockBytes;
-  const uint8_t* wg = a.gate + (size_t)e * a.expert_bytes;
-  const uint8_t* wu = a.up + (size_t)e * a.expert_bytes;
   const int wave_row0 = (tile * kWavesPerWg + wave) * DEPTH * RPS;
-  Raw r[DEPTH][2];
-#pragma unroll
-  for (int d = 0; d < DEPTH; ++d) {
-    const int row0 = wave_row0 + d * RPS;  // the tiles divide the rows exactly (checked by the host)
-    load_raw<RQ>(wg + (size_t)row0 * row_bytes, true, g, r[d][0]);
-    load_raw<RQ>(wu + (size_t)row0 * row_bytes, true, g, r[d][1]);
-  }
   float* out = a.inter + (size_t)p * a.I;
+  // the pair's rows of expert e: all loads, (the routing wavefront: the rest of the routing,) accumulation
+  auto stream_rows = [&](int e, auto finish_c) __attribute__((always_inline)) {
+    constexpr bool kFinish = decltype(finish_c)::value;
+    const uint8_t* wg = a.gate + (size_t)e * a.expert_bytes;
+    const uint8_t* wu = a.up + (size_t)e * a.expert_bytes;
+    Raw r[DEPTH][2];
+    auto request = [&](int d0, int d1) __attribute__((always_inline)) {
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) {
-    if (d == 1) XABE_TRACE(1, 2);
-    float tg[1] = {0.0f}, tu[1] = {0.0f};
-    accum<RQ, 1>(r[d][0], g, x, xs, tg);
-    accum<RQ, 1>(r[d][1], g, x, xs, tu);
-    const float sg = group_sum<G>(tg[0]), su = group_sum<G>(tu[0]);
-    const int row = wave_row0 + d * RPS + g.lane / G;
-    if ((g.lane % G) == 0 && row < a.I) out[row] = silu_f(sg) * su;
-  }
+      for (int d = 0; d < DEPTH; ++d) {
+        if (d < d0 || d >= d1) continue;
+        const int row0 = wave_row0 + d * RPS;  // the tiles divide the rows exactly (checked by the host)
+        load_raw<RQ>(wg + (size_t)row0 * row_bytes, true, g, r[d][0]);
+        load_raw<RQ>(wu + (size_t)row0 * row_bytes, true, g, r[d][1]);
+      }
+    };
+    // The routing wavefront finishes the softmax before it requests its own rows: its neighbours' requests
+    // fill the CU's memory pipeline at this point, and a load issued now would hold the wavefront (and the
+    // routing) until they drain; raised priority keeps it ahead of their arithmetic.
+    if constexpr (kFinish) {
+      if (routes) {
+        __builtin_amdgcn_s_setprio(3);
+        int sel_i;
+        float sel_w;
+        bool exact;
+        if (few) route_finish<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, a.top_k, n_cand, cand_i, s_route, sel_i, sel_w, exact);
+        else route_finish<kRouteMaxPerLane>(lg, a.E, a.top_k, n_cand, cand_i, s_route, sel_i, sel_w, exact);
+        XABE_ROUTE_TRACE(5);
+        if (g.lane == k) s_final = sel_i;
+        if (k == 0 && tile == 0 && g.lane < a.top_k) {
+          a.topk_ids[(size_t)t * a.top_k + g.lane] = sel_i;
+          a.topk_weights[(size_t)t * a.top_k + g.lane] = sel_w;
+        }
+        __builtin_amdgcn_s_setprio(0);
+      }
+    }
+    request(0, DEPTH);  // (the other wavefronts come straight here)
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (d == 1) XABE_TRACE(1, 2);
+      float tg[1] = {0.0f}, tu[1] = {0.0f};
+      accum<RQ, 1>(r[d][0], g, x, xs, tg);
+      accum<RQ, 1>(r[d][1], g, x, xs, tu);
+      const float sg = group_sum<G>(tg[0]), su = group_sum<G>(tu[0]);
+      const int row = wave_row0 + d * RPS + g.lane / G;
+      if ((g.lane % G) == 0 && row < a.I) out[row] = silu_f(sg) * su;
+    }
+  };
+  const int e = s_expert;
+  stream_rows(e, std::true_type{});
+  __syncthreads();  // s_final is there
+  const int e_final = s_final;
+  if (e_final != e) stream_rows(e_final, std::false_type{});  // (same rows of `inter`, written again)
   XABE_TRACE(1, 3);
 }
 

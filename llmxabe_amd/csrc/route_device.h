@@ -38,9 +38,59 @@ __device__ __forceinline__ void route_load(const float* lg, int num_experts, con
   }
 }
 
+// One selection round over per-lane keys (kTaken = out of the running): the largest key, the lowest index
+// among equals; the winner is marked taken.  Returns the winning key and index to every lane.
+constexpr int kRouteTaken = (int)0x80000000;
 template <int PER>
-__device__ __forceinline__ void route_compute(const float (&l)[PER], int num_experts, int top_k, float* e_all,
-                                              int& sel_i, float& sel_w) {
+__device__ __forceinline__ void route_round(int (&key)[PER], int& best, int& bi) {
+  const int lane = threadIdx.x & 63;
+  int bp = key[0];
+#pragma unroll
+  for (int i = 1; i < PER; ++i) bp = max(bp, key[i]);
+  best = wave_max_i(bp);
+  int li = 0x7fffffff;
+#pragma unroll
+  for (int i = PER - 1; i >= 0; --i)
+    if (key[i] == best) li = i * 64 + lane;  // descending i: the lowest index of this lane wins
+  const unsigned long long holders = __builtin_amdgcn_ballot_w64(li != 0x7fffffff);
+  if (__builtin_popcountll(holders) == 1) bi = __builtin_amdgcn_readlane(li, __builtin_ctzll(holders));
+  else bi = wave_min_i(li);
+  if ((bi & 63) == lane) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (i == (bi >> 6)) key[i] = kRouteTaken;
+  }
+}
+
+// First half of route_compute: the n experts with the largest LOGITS, in order (lower index first among
+// equal logits); lane j < n returns the j-th in cand_i.  exp and the division by the common sum are
+// monotone non-decreasing, so p orders the experts the same way except where distinct logits round to the
+// same p: with n = top_k + 1 candidates, route_finish sees whether that happened anywhere it matters, and
+// the candidates are then the selection itself -- known before a single exp has been evaluated.
+template <int PER>
+__device__ __forceinline__ void route_order(const float (&l)[PER], int num_experts, int n, int& cand_i) {
+  const int lane = threadIdx.x & 63;
+  int key[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int b = __builtin_bit_cast(int, l[i]);
+    key[i] = i * 64 + lane < num_experts ? b ^ ((b >> 31) & 0x7fffffff) : kRouteTaken;  // int order == float order
+  }
+  cand_i = 0;
+  for (int j = 0; j < n; ++j) {
+    int best, bi;
+    route_round<PER>(key, best, bi);
+    if (lane == j) cand_i = bi;
+  }
+}
+
+// Second half: softmax, then the selection.  If the top_k + 1 candidates' probabilities are strictly
+// decreasing (lane j against lane j + 1, j < top_k) the candidates are the reference's selection; otherwise
+// some probabilities tie and the selection is redone on the probabilities themselves, the reference's way.
+// `exact` (wave-uniform) tells the caller whether cand_i stood.
+template <int PER>
+__device__ __forceinline__ void route_finish(const float (&l)[PER], int num_experts, int top_k, int n, int cand_i,
+                                             float* e_all, int& sel_i, float& sel_w, bool& exact) {
   const int lane = threadIdx.x & 63;
   float m = l[0];
 #pragma unroll
@@ -78,36 +128,26 @@ __device__ __forceinline__ void route_compute(const float (&l)[PER], int num_exp
   }
   sum = lane_bcast(sum, 0);
   XABE_ROUTE_TRACE(3);
-  // p >= +0, so the bit patterns order like the values and the selection runs on integers (one DPP
-  // max per reduction step, no NaN canonicalisation); kTaken marks entries that are out of the running
-  constexpr int kTaken = -1;
-  int p[PER];
+  // p >= +0, so the bit patterns order like the values and comparisons run on integers
+  const int pj = lane < n ? __builtin_bit_cast(int, e_all[cand_i] / sum) : 0;
+  const int pn = __builtin_amdgcn_ds_bpermute(((lane + 1) & 63) * 4, pj);
+  const bool strict = lane >= top_k || lane + 1 >= n || pj > pn;
+  exact = __builtin_amdgcn_ballot_w64(strict) == ~0ull;
+  int sel_bits = pj;
+  sel_i = cand_i;
+  if (!exact) {
+    int p[PER];
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const int idx = i * 64 + lane;
-    p[i] = idx < num_experts ? __builtin_bit_cast(int, e_all[idx] / sum) : kTaken;
-  }
-  // top-k: each round takes the largest p not yet taken, the lowest index among equals
-  int sel_bits = 0;
-  sel_i = 0;
-  for (int k = 0; k < top_k; ++k) {
-    int bp = p[0];
-#pragma unroll
-    for (int i = 1; i < PER; ++i) bp = max(bp, p[i]);
-    const int best = wave_max_i(bp);
-    int li = 0x7fffffff;
-#pragma unroll
-    for (int i = PER - 1; i >= 0; --i)
-      if (p[i] == best) li = i * 64 + lane;  // descending i: the lowest index of this lane wins
-    const unsigned long long holders = __builtin_amdgcn_ballot_w64(li != 0x7fffffff);
-    int bi;
-    if (__builtin_popcountll(holders) == 1) bi = __builtin_amdgcn_readlane(li, __builtin_ctzll(holders));
-    else bi = wave_min_i(li);
-    if (lane == k) { sel_bits = best; sel_i = bi; }
-    if ((bi & 63) == lane) {
-#pragma unroll
-      for (int i = 0; i < PER; ++i)
-        if (i == (bi >> 6)) p[i] = kTaken;
+    for (int i = 0; i < PER; ++i) {
+      const int idx = i * 64 + lane;
+      p[i] = idx < num_experts ? __builtin_bit_cast(int, e_all[idx] / sum) : kRouteTaken;
+    }
+    sel_bits = 0;
+    sel_i = 0;
+    for (int k = 0; k < top_k; ++k) {
+      int best, bi;
+      route_round<PER>(p, best, bi);
+      if (lane == k) { sel_bits = best; sel_i = bi; }
     }
   }
   const float sel_p = __builtin_bit_cast(float, sel_bits);
@@ -116,6 +156,16 @@ __device__ __forceinline__ void route_compute(const float (&l)[PER], int num_exp
   float ssum = -0.0f;
   for (int k = 0; k < top_k; ++k) ssum += lane_bcast(sel_p, k);
   sel_w = ssum > 0.0f ? sel_p / ssum : 1.0f / (float)top_k;
+}
+
+template <int PER>
+__device__ __forceinline__ void route_compute(const float (&l)[PER], int num_experts, int top_k, float* e_all,
+                                              int& sel_i, float& sel_w) {
+  const int n = min(top_k + 1, num_experts);
+  int cand_i;
+  bool exact;
+  route_order<PER>(l, num_experts, n, cand_i);
+  route_finish<PER>(l, num_experts, top_k, n, cand_i, e_all, sel_i, sel_w, exact);
 }
 
 template <bool COHERENT = false>

@@ -102,6 +102,35 @@ def test_model_geometry_f32_router(oracle, X):
     _compare(X, oracle, g, (3, 2), seed=4400, router_q8=False)
 
 
+def test_candidate_expert_replaced_after_verification(oracle, X):
+    """Launch B starts streaming the expert ranked k-th by LOGIT and re-streams when the probabilities rank
+    another one there.  A zero router with a crafted bias gives logits = bias exactly: two experts one ulp
+    apart whose probabilities tie, the larger logit at the higher index, inside the top 8 and across ranks
+    8 / 9, so the pairs k = 1, 2 and 7 of every token change expert after the softmax."""
+    import torch
+
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(3), 3)
+    layer = make_layer(oracle, g, seed=4600, router_q8=False)
+    layer.dev.router.zero_()
+    bias = np.random.default_rng(5).uniform(-8.0, -1.0, 256).astype(np.float32)
+    bias[50] = 5.0
+    bias[10], bias[200] = 0.001, np.nextafter(np.float32(0.001), np.float32(1))
+    bias[120:124] = (-0.1, -0.2, -0.3, -0.4)
+    bias[30], bias[220] = -0.5, np.nextafter(np.float32(-0.5), np.float32(0))
+    lb = torch.from_numpy(bias).cuda()
+    one, many = X.MoeBlock(g), X.MoeBlock(g)
+    many.set_fused_decode(False)
+    x = activations(4610, 3, 2048)
+    f1, l1 = run_block(one, layer, x, 3, logit_bias=lb)
+    f2, l2 = run_block(many, layer, x, 3, logit_bias=lb)
+    a, b = _observe(one, g, f1, l1, 3), _observe(many, g, f2, l2, 3)
+    ref_ids, _ = oracle.route_batch(np.tile(bias, (3, 1)), 8)
+    assert list(ref_ids[0]) == [50, 10, 200, 120, 121, 122, 123, 30]
+    assert np.array_equal(a["logits"], np.tile(bias, (3, 1)))
+    assert np.array_equal(a["ids"], ref_ids.astype(np.int32))
+    _same_bits(a, b, "near-tie routing")
+
+
 def test_many_replays_keep_the_bits(oracle, X):
     # 200 back-to-back passes on one stream, no host work between
     import torch

@@ -102,6 +102,32 @@ def test_route_all_tie_selects_lowest_indices(oracle, X):
         assert np.allclose(b.topk_weights().cpu().numpy().reshape(8, 8)[:5], 0.125)
 
 
+def _near_tie_logits(rows=6, seed=21):
+    """Logits whose order disagrees with (probability desc, index asc): pairs one ulp apart, the larger at the
+    HIGHER index, far enough below the row maximum that l - max rounds both to the same value.  One pair sits
+    inside the top 8, one straddles ranks 8 and 9 (the reference keeps the lower index of each)."""
+    rng = np.random.default_rng(seed)
+    logits = rng.uniform(-8.0, -1.0, (rows, 256)).astype(np.float32)
+    for r in range(rows):
+        logits[r, 50 + r] = 5.0
+        logits[r, 10], logits[r, 200] = 0.001, np.nextafter(np.float32(0.001), np.float32(1))
+        logits[r, 120:124] = (-0.1, -0.2, -0.3, -0.4)
+        logits[r, 30], logits[r, 220] = -0.5, np.nextafter(np.float32(-0.5), np.float32(0))
+    return logits
+
+
+def test_route_near_ties_fall_back_to_the_probability_order(oracle, X):
+    logits = _near_tie_logits()
+    ref_ids, ref_w = oracle.route_batch(logits, 8)
+    # the construction does what it says: ranking by logit alone would pick 200 before 10, and 220 not 30
+    assert list(ref_ids[0][:3]) == [50, 10, 200] and ref_ids[0][7] == 30 and 220 not in ref_ids[0]
+    k, b, g = _route(X, logits, 8, 6)
+    ids = b.topk_ids().cpu().numpy().reshape(8, 8)
+    w = b.topk_weights().cpu().numpy().reshape(8, 8)
+    assert np.array_equal(ids[:6], ref_ids.astype(np.int32))
+    assert np.abs(w[:6] - ref_w).max() <= 1.2e-7
+
+
 def test_route_many_tokens_and_extreme_logits(oracle, X):
     rng = np.random.default_rng(9)
     logits = (rng.standard_normal((512, 256)) * 3).astype(np.float32)
