@@ -42,7 +42,29 @@ typedef enum xabe_status {
   XABE_ERR_BUFFER_LENGTH = 9,         /* MoeBlockError::BufferLength { what, expected, found } */
   XABE_ERR_INVALID_ARGUMENT = 10,     /* a NULL handle or pointer (the Rust API rules this out by type) */
   XABE_ERR_UNSUPPORTED_QUANT = 11,    /* MoeBlockError::UnsupportedExpertType: Q4_0/Q4_K/Q5_K have no kernel here */
-  XABE_ERR_FFN_KIND_MISMATCH = 12     /* MoeBlockError::FfnKindMismatch */
+  XABE_ERR_FFN_KIND_MISMATCH = 12,    /* MoeBlockError::FfnKindMismatch */
+  XABE_ERR_MISSING_TENSOR = 13,       /* MoeBlockError::MissingTensor { role, layer } */
+  XABE_ERR_UNSUPPORTED_DENSE_TYPE = 14, /* MoeBlockError::UnsupportedDenseType { name, found } */
+  XABE_ERR_SHAPE_MISMATCH = 15,       /* MoeBlockError::ShapeMismatch { name, expected, found } */
+  /* GgufError (crates/xabe-gguf/src/error.rs:11-108), one status per variant */
+  XABE_ERR_GGUF_BAD_MAGIC = 20,
+  XABE_ERR_GGUF_UNSUPPORTED_VERSION = 21,
+  XABE_ERR_GGUF_UNEXPECTED_EOF = 22,
+  XABE_ERR_GGUF_INVALID_UTF8 = 23,
+  XABE_ERR_GGUF_NEGATIVE_COUNT = 24,
+  XABE_ERR_GGUF_DUPLICATE_KEY = 25,
+  XABE_ERR_GGUF_UNKNOWN_VALUE_TYPE = 26,
+  XABE_ERR_GGUF_NESTED_ARRAY = 27,
+  XABE_ERR_GGUF_BAD_ALIGNMENT_TYPE = 28,
+  XABE_ERR_GGUF_BAD_ALIGNMENT = 29,
+  XABE_ERR_GGUF_TOO_MANY_DIMENSIONS = 30,
+  XABE_ERR_GGUF_ZERO_DIMENSION = 31,
+  XABE_ERR_GGUF_DUPLICATE_TENSOR = 32,
+  XABE_ERR_GGUF_UNSUPPORTED_GGML_TYPE = 33,
+  XABE_ERR_GGUF_UNALIGNED_ELEMENT_COUNT = 34,
+  XABE_ERR_GGUF_OFFSET_OVERFLOW = 35,
+  XABE_ERR_GGUF_TENSOR_OUT_OF_BOUNDS = 36,
+  XABE_ERR_GGUF_IO = 37
 } xabe_status;
 
 const char* xabe_last_error(void);

@@ -3,3 +3,4 @@ from .moe import (BLOCK_Q6_K_DEVICE_BYTES, BufferScope, ExpertQuant, LayerOpsKer
                   MoeGeometry, MoeKernels, QuantTensor, calibrate_hbm_read, calibrate_mfma_f16, dequantize, moe_block_size,
                   synth_normal_f32, synth_quant, to_device_layout)
 from .block import DEFAULT_RMS_EPS, DenseFfnBlock, DenseFfnLayerWeights, MoeBlock, MoeLayerWeights  # noqa: F401
+from .gguf import GgmlType, GgufError, GgufFile, TensorInfo, UploadedDenseFfnLayer, UploadedMoeLayer  # noqa: F401

@@ -10,6 +10,8 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libxabe_hip.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "xabe_hip.h")
+GGUF_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "xabe_gguf.h")
+HEADER_PATHS = (HEADER_PATH, GGUF_HEADER_PATH)
 
 sz = C.c_size_t
 vp = C.c_void_p
@@ -34,6 +36,14 @@ class MoeLayerWeightsC(C.Structure):
 class DenseLayerWeightsC(C.Structure):
     _fields_ = [("post_norm", vp), ("gate", QuantTensorC), ("up", QuantTensorC), ("down", QuantTensorC)]
 
+
+class TensorInfoC(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("n_dims", C.c_uint32), ("dims", C.c_uint64 * 4), ("ggml_type", C.c_int),
+                ("offset", C.c_uint64), ("n_elements", C.c_uint64), ("n_bytes", C.c_uint64)]
+
+
+u64 = C.c_uint64
+cp = C.c_char_p
 
 _SIGNATURES = {
     "xabe_last_error": (C.c_char_p, []),
@@ -112,6 +122,43 @@ _SIGNATURES = {
     "xabe_calibrate_hbm_read": (C.c_int, [vp, vp, sz, vp]),
     "xabe_calibrate_mfma_f16": (C.c_int, [vp, vp, sz, C.c_int, C.POINTER(C.c_double)]),
     "xabe_synth_quant": (C.c_int, [vp, C.c_int, C.c_uint64, sz, C.c_float, vp, sz]),
+    # include/xabe_gguf.h
+    "xabe_ggml_type_block_size": (u64, [C.c_int]),
+    "xabe_ggml_type_size": (u64, [C.c_int]),
+    "xabe_ggml_type_name": (cp, [C.c_int]),
+    "xabe_ggml_type_bytes_for_elements": (C.c_int, [C.c_int, u64, C.POINTER(u64)]),
+    "xabe_gguf_open": (C.c_int, [cp, C.POINTER(vp)]),
+    "xabe_gguf_from_bytes": (C.c_int, [vp, sz, C.POINTER(vp)]),
+    "xabe_gguf_close": (None, [vp]),
+    "xabe_gguf_version": (C.c_uint32, [vp]),
+    "xabe_gguf_alignment": (C.c_uint32, [vp]),
+    "xabe_gguf_n_kv": (sz, [vp]),
+    "xabe_gguf_n_tensors": (sz, [vp]),
+    "xabe_gguf_data_offset": (u64, [vp]),
+    "xabe_gguf_tensor_at": (C.c_int, [vp, sz, C.POINTER(TensorInfoC)]),
+    "xabe_gguf_tensor": (C.c_int, [vp, cp, C.POINTER(TensorInfoC)]),
+    "xabe_gguf_tensor_bytes": (vp, [vp, cp, C.POINTER(sz)]),
+    "xabe_gguf_key_at": (cp, [vp, sz]),
+    "xabe_gguf_value_type_of": (C.c_int, [vp, cp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(u64)]),
+    "xabe_gguf_get_u32": (C.c_int, [vp, cp, C.POINTER(C.c_uint32)]),
+    "xabe_gguf_get_u64": (C.c_int, [vp, cp, C.POINTER(u64)]),
+    "xabe_gguf_get_f32": (C.c_int, [vp, cp, C.POINTER(C.c_float)]),
+    "xabe_gguf_get_str": (vp, [vp, cp, C.POINTER(sz)]),
+    "xabe_gguf_get_array": (vp, [vp, cp, C.c_int, C.POINTER(u64)]),
+    "xabe_gguf_get_string_array_item": (vp, [vp, cp, u64, C.POINTER(sz)]),
+    "xabe_moe_layer_upload": (C.c_int, [vp, vp, C.c_uint32, C.POINTER(Geometry), C.POINTER(vp)]),
+    "xabe_moe_layer_free": (None, [vp]),
+    "xabe_moe_layer_weights_of": (C.POINTER(MoeLayerWeightsC), [vp]),
+    "xabe_moe_layer_index": (C.c_uint32, [vp]),
+    "xabe_moe_layer_expert_quants": (C.c_int, [vp, C.POINTER(C.c_int * 3)]),
+    "xabe_moe_layer_shared_quants": (C.c_int, [vp, C.POINTER(C.c_int * 3)]),
+    "xabe_moe_layer_router_types": (C.c_int, [vp, C.POINTER(C.c_int * 2)]),
+    "xabe_moe_layer_bytes": (sz, [vp]),
+    "xabe_dense_ffn_layer_upload": (C.c_int, [vp, vp, C.c_uint32, sz, sz, C.POINTER(vp)]),
+    "xabe_dense_ffn_layer_free": (None, [vp]),
+    "xabe_dense_ffn_layer_weights_of": (C.POINTER(DenseLayerWeightsC), [vp]),
+    "xabe_dense_ffn_layer_quants": (C.c_int, [vp, C.POINTER(C.c_int * 3)]),
+    "xabe_dense_ffn_layer_bytes": (sz, [vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

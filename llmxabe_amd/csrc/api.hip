@@ -274,6 +274,27 @@ const char* xabe_status_name(int s) {
     case XABE_ERR_INVALID_ARGUMENT: return "InvalidArgument";
     case XABE_ERR_UNSUPPORTED_QUANT: return "UnsupportedExpertType";
     case XABE_ERR_FFN_KIND_MISMATCH: return "FfnKindMismatch";
+    case XABE_ERR_MISSING_TENSOR: return "MissingTensor";
+    case XABE_ERR_UNSUPPORTED_DENSE_TYPE: return "UnsupportedDenseType";
+    case XABE_ERR_SHAPE_MISMATCH: return "ShapeMismatch";
+    case XABE_ERR_GGUF_BAD_MAGIC: return "BadMagic";
+    case XABE_ERR_GGUF_UNSUPPORTED_VERSION: return "UnsupportedVersion";
+    case XABE_ERR_GGUF_UNEXPECTED_EOF: return "UnexpectedEof";
+    case XABE_ERR_GGUF_INVALID_UTF8: return "InvalidUtf8";
+    case XABE_ERR_GGUF_NEGATIVE_COUNT: return "NegativeCount";
+    case XABE_ERR_GGUF_DUPLICATE_KEY: return "DuplicateKey";
+    case XABE_ERR_GGUF_UNKNOWN_VALUE_TYPE: return "UnknownValueType";
+    case XABE_ERR_GGUF_NESTED_ARRAY: return "NestedArray";
+    case XABE_ERR_GGUF_BAD_ALIGNMENT_TYPE: return "BadAlignmentType";
+    case XABE_ERR_GGUF_BAD_ALIGNMENT: return "BadAlignment";
+    case XABE_ERR_GGUF_TOO_MANY_DIMENSIONS: return "TooManyDimensions";
+    case XABE_ERR_GGUF_ZERO_DIMENSION: return "ZeroDimension";
+    case XABE_ERR_GGUF_DUPLICATE_TENSOR: return "DuplicateTensor";
+    case XABE_ERR_GGUF_UNSUPPORTED_GGML_TYPE: return "UnsupportedGgmlType";
+    case XABE_ERR_GGUF_UNALIGNED_ELEMENT_COUNT: return "UnalignedElementCount";
+    case XABE_ERR_GGUF_OFFSET_OVERFLOW: return "OffsetOverflow";
+    case XABE_ERR_GGUF_TENSOR_OUT_OF_BOUNDS: return "TensorOutOfBounds";
+    case XABE_ERR_GGUF_IO: return "Io";
   }
   return "Unknown";
 }

@@ -9,7 +9,7 @@ import pytest
 def _header_functions():
     from llmxabe_amd import _ffi
 
-    src = open(_ffi.HEADER_PATH).read()
+    src = "".join(open(p).read() for p in _ffi.HEADER_PATHS)
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
     return sorted(set(re.findall(r"\b(xabe_[a-z0-9_]+)\s*\(", src)))
 
