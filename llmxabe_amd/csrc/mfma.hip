@@ -120,9 +120,8 @@ __device__ __forceinline__ void load_step_a(int ks, const _Float16* const (&arow
 }
 // ... and the raw blocks of this thread's two weight-row units.
 template <int QUANT>
-__device__ __forceinline__ void load_step_w(int ks, const uint8_t* const (&wrow)[2], int du, WRaw<QUANT>& wreg) {
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
+__device__ __forceinline__ void load_unit_w(int ks, int i, const uint8_t* const (&wrow)[2], int du, WRaw<QUANT>& wreg) {
+  {
     if constexpr (QUANT == kQ6K) {
       // step ks covers half (ks & 1) of superblock ks >> 1
       const uint8_t* p = wrow[i] + (size_t)(ks >> 1) * kQ6KBytes;
@@ -135,6 +134,23 @@ __device__ __forceinline__ void load_step_w(int ks, const uint8_t* const (&wrow)
     }
   }
 }
+template <int QUANT>
+__device__ __forceinline__ void load_step_w(int ks, const uint8_t* const (&wrow)[2], int du, WRaw<QUANT>& wreg) {
+  load_unit_w<QUANT>(ks, 0, wrow, du, wreg);
+  load_unit_w<QUANT>(ks, 1, wrow, du, wreg);
+}
+
+#ifdef XABE_MFMA_TRACE
+// measurement builds only: [workgroup < 512][step slot < 32][4 stamps] of the routed gate/up launch (100 MHz clock)
+static __device__ long long g_mfma_trace[512 * 32 * 4];
+#define XABE_MT(slot)                                                                                             \
+  do {                                                                                                            \
+    if (NM == 2 && ROUTED && tid == 0 && blockIdx.x < 512 && trace_step < 32)                                     \
+      g_mfma_trace[(blockIdx.x * 32 + trace_step) * 4 + (slot)] = wall_clock64();                                 \
+  } while (0)
+#else
+#define XABE_MT(slot) do { } while (0)
+#endif
 
 template <int QUANT, int NM, bool ROUTED>
 __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
@@ -158,8 +174,20 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   // dequant mapping: unit u of LDS weight rows rb0 and rb0 + 64
   const int du = tid & 3, rb0 = tid >> 2;
 
-  for (int item = blockIdx.x; item < total; item += gridDim.x) {
-    const int mt = item / n_ntiles, nt = item % n_ntiles;
+  [[maybe_unused]] int trace_step = 0;
+  // Which items this workgroup takes.  Workgroup ids are dealt round-robin to the eight XCDs, each with its
+  // own L2: when there is work for every workgroup, XCD x takes a contiguous eighth of the token tiles and its
+  // workgroups walk that range together (token tile major), so an activation tile is fetched into one L2
+  // once instead of into all eight, and the token tiles of one expert reuse its weights from that L2.
+  const bool by_xcd = (gridDim.x & 7u) == 0 && total >= 2 * (int)gridDim.x && n_mtiles >= 8;
+  const int xcd = blockIdx.x & 7;
+  const int m_lo = by_xcd ? (int)((long long)n_mtiles * xcd / 8) : 0;
+  const int m_hi = by_xcd ? (int)((long long)n_mtiles * (xcd + 1) / 8) : n_mtiles;
+  const int first = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int stride = by_xcd ? (int)(gridDim.x >> 3) : (int)gridDim.x;
+  const int local_total = (m_hi - m_lo) * n_ntiles;
+  for (int item = first; item < local_total; item += stride) {
+    const int mt = m_lo + item / n_ntiles, nt = item % n_ntiles;
     int e = 0, m0 = mt * kBM, rows = min(kBM, valid - mt * kBM);
     if (ROUTED) {
       e = a.tile_list[4 + 4 * mt];
@@ -232,6 +260,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     auto step = [&](auto p_c, int ks) __attribute__((always_inline)) {
       constexpr int P = decltype(p_c)::value % kWDepth;
       __syncthreads();  // everyone has finished reading the previous step's tiles
+      XABE_MT(0);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int c = tid + 256 * i;
@@ -243,22 +272,39 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
         if constexpr (QUANT == kQ6K) q6_unit_to_lds(w[P].u[i], du, &sB[rb * kLd]);
         else q8_unit_to_lds(w[P].u[i], &sB[rb * kLd + du * 32]);
       }
+      XABE_MT(1);
       __syncthreads();
+      XABE_MT(2);
       if (ks + 1 < nks) load_step_a(ks + 1, arow_ptr, areg);  // in flight while the matrix cores work
       if (ks + kWDepth < nks) load_step_w<QUANT>(ks + kWDepth, wrow, du, w[P]);
       const _Float16* pa = &sA[(wm * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
       const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
+      // Operand fragments one sub-step ahead, in two register sets: the four LDS reads of sub-step kk + 1 are
+      // issued before the four matrix instructions of sub-step kk, so their latency hides behind 128 cycles of
+      // matrix work instead of standing between every group of four.
+      half8 fa[2][2], fb[2][2];
+      auto frags = [&](int kk, int set) __attribute__((always_inline)) {
+        fa[set][0] = *reinterpret_cast<const half8*>(pa + kk * 16);
+        fa[set][1] = *reinterpret_cast<const half8*>(pa + 32 * kLd + kk * 16);
+        fb[set][0] = *reinterpret_cast<const half8*>(pb + kk * 16);
+        fb[set][1] = *reinterpret_cast<const half8*>(pb + 32 * kLd + kk * 16);
+      };
+      frags(0, 0);
 #pragma unroll
       for (int kk = 0; kk < kBK / 16; ++kk) {
-        const half8 a0 = *reinterpret_cast<const half8*>(pa + kk * 16);
-        const half8 a1 = *reinterpret_cast<const half8*>(pa + 32 * kLd + kk * 16);
-        const half8 b0 = *reinterpret_cast<const half8*>(pb + kk * 16);
-        const half8 b1 = *reinterpret_cast<const half8*>(pb + 32 * kLd + kk * 16);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b0, acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b1, acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b0, acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc[1][1], 0, 0, 0);
+        const int c = kk & 1;
+        if (kk + 1 < kBK / 16) frags(kk + 1, c ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][0], fb[c][0], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][0], fb[c][1], acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][1], fb[c][0], acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][1], fb[c][1], acc[1][1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
+      XABE_MT(3);
+#ifdef XABE_MFMA_TRACE
+      ++trace_step;
+#endif
     };
     if constexpr (kWDepth == 2) {
       for (int ks = 0; ks < nks; ks += 2) {
@@ -451,3 +497,9 @@ int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffer
 }
 
 }  // namespace xabe
+
+#ifdef XABE_MFMA_TRACE
+extern "C" int xabe_debug_read_mfma_trace(long long* out, size_t n) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(xabe::g_mfma_trace), n * sizeof(long long));
+}
+#endif
