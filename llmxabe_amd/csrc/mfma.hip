@@ -154,10 +154,12 @@ static __device__ long long g_mfma_trace[512 * 32 * 4];
 
 template <int QUANT, int NM, bool ROUTED>
 __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
-  // 71 KB of LDS per workgroup (two per CU): dynamic, since the static limit is 64 KB
+  // 72.5 KB of LDS per workgroup (two per CU): dynamic, since the static limit is 64 KB
   extern __shared__ __attribute__((aligned(16))) uint8_t mfma_smem[];
   _Float16* sA = reinterpret_cast<_Float16*>(mfma_smem);
   _Float16* sB = sA + kBM * kLd;
+  // row tables, two sets (this item's and the next one's), each kTable = 3 * kBM words apart
+  constexpr int kTable = 3 * kBM;
   int* sArow = reinterpret_cast<int*>(sB + kBR * kLd);  // activation row index of each tile row
   int* sOrow = sArow + kBM;                             // output row index, or -1 for a dead row
   float* sScale = reinterpret_cast<float*>(sOrow + kBM);
@@ -186,36 +188,40 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   const int first = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
   const int stride = by_xcd ? (int)(gridDim.x >> 3) : (int)gridDim.x;
   const int local_total = (m_hi - m_lo) * n_ntiles;
-  for (int item = first; item < local_total; item += stride) {
-    const int mt = m_lo + item / n_ntiles, nt = item % n_ntiles;
-    int e = 0, m0 = mt * kBM, rows = min(kBM, valid - mt * kBM);
-    if (ROUTED) {
-      e = a.tile_list[4 + 4 * mt];
-      m0 = a.tile_list[4 + 4 * mt + 1];
-      rows = a.tile_list[4 + 4 * mt + 2];
-    }
-    __syncthreads();  // the previous item is done with the row tables
-    if (tid < kBM) {
-      int arow = 0, orow = -1;
-      float sc = 1.0f;
-      if (tid < rows) {
-        if (ROUTED) {
-          const int slot = m0 + tid;
-          const int flat = a.sorted_token_ids[slot];
-          if (NM == 2) { arow = flat / a.top_k; orow = slot; }
-          else { arow = slot; orow = flat; sc = a.topk_weights[flat]; }
-        } else {
-          arow = orow = m0 + tid;
-        }
-      }
-      sArow[tid] = arow;
-      sOrow[tid] = orow;
-      sScale[tid] = sc;
-    }
-    __syncthreads();
+  if (first >= local_total) return;
 
-    // weight rows this thread dequantises
-    const uint8_t* wrow[2];
+  // One item = (token tile, weight-row tile).  Items are pipelined: the row tables, pointers and first loads of
+  // item i + 1 are set up inside the last contraction step of item i, so its epilogue and the latency of the
+  // next item's first loads overlap instead of adding up (the weight loads of a short contraction, 4 steps
+  // for the down projection, otherwise wait ~8 us per item with nothing to hide behind).
+  struct Item { int e, m0, rows, nt; };
+  auto decode = [&](int item) __attribute__((always_inline)) {
+    const int mt = m_lo + item / n_ntiles;
+    Item it{0, mt * kBM, min(kBM, valid - mt * kBM), item % n_ntiles};
+    if (ROUTED) {
+      it.e = a.tile_list[4 + 4 * mt];
+      it.m0 = a.tile_list[4 + 4 * mt + 1];
+      it.rows = a.tile_list[4 + 4 * mt + 2];
+    }
+    return it;
+  };
+  // table entry of tile row `tid` (threads below kBM): activation row, output row (-1: dead), output scale
+  auto table_entry = [&](const Item& it, int& arow, int& orow, float& sc) __attribute__((always_inline)) {
+    arow = 0, orow = -1, sc = 1.0f;
+    if (tid < it.rows) {
+      if (ROUTED) {
+        const int slot = it.m0 + tid;
+        const int flat = a.sorted_token_ids[slot];
+        if (NM == 2) { arow = flat / a.top_k; orow = slot; }
+        else { arow = slot; orow = flat; sc = a.topk_weights[flat]; }
+      } else {
+        arow = orow = it.m0 + tid;
+      }
+    }
+  };
+  const uint8_t* wrow[2];        // weight rows this thread dequantises
+  const _Float16* arow_ptr[8];   // activation chunks this thread stages: 8 x 16 bytes per step
+  auto set_wrow = [&](const Item& it) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int rb = rb0 + 64 * i;
@@ -224,20 +230,55 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       if (NM == 2) {
         const int half_n = rb >> 6, which = (rb >> 5) & 1, c = rb & 31;
         base = which ? a.w1 : a.w0;
-        wr = nt * 64 + half_n * 32 + c;
+        wr = it.nt * 64 + half_n * 32 + c;
       } else {
         base = a.w0;
-        wr = nt * 128 + rb;
+        wr = it.nt * 128 + rb;
       }
-      wrow[i] = base + (size_t)e * a.expert_bytes + (size_t)wr * row_bytes;
+      wrow[i] = base + (size_t)it.e * a.expert_bytes + (size_t)wr * row_bytes;
     }
-    // activation chunks this thread stages: 8 x 16 bytes per step
-    const _Float16* arow_ptr[8];
+  };
+  auto set_arow = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int c = tid + 256 * i;
-      arow_ptr[i] = a.a + (size_t)sArow[c >> 4] * a.K + (c & 15) * 8;
+      arow_ptr[i] = a.a + (size_t)sArow[buf * kTable + (c >> 4)] * a.K + (c & 15) * 8;
     }
+  };
+
+  // In flight per step: the next step's activation chunks (one matrix phase ahead: they come from L2) and the
+  // raw weight bytes of the next two steps (the HBM-cold ones), in w[ks & 1].  The contraction has an even
+  // number of steps (whole superblocks), so the step pairs are unrolled and no register is copied.
+  // (The down launch, NM = 1, has no registers to spare for the second step and keeps one in flight.)
+  constexpr int kWDepth = NM == 2 ? 2 : 1;
+  u32x4 areg[8];
+  WRaw<QUANT> w[kWDepth];
+
+  Item cur = decode(first);
+  {
+    int arow, orow;
+    float sc;
+    if (tid < kBM) {
+      table_entry(cur, arow, orow, sc);
+      sArow[tid] = arow;
+      sOrow[tid] = orow;
+      sScale[tid] = sc;
+    }
+    __syncthreads();
+    set_wrow(cur);
+    set_arow(0);
+    load_step_w<QUANT>(0, wrow, du, w[0]);
+    load_step_a(0, arow_ptr, areg);
+    if constexpr (kWDepth == 2) load_step_w<QUANT>(1, wrow, du, w[kWDepth - 1]);
+  }
+  int buf = 0;
+  for (int item = first;; item += stride) {
+    const bool has_next = item + stride < local_total;
+    const Item nxt = has_next ? decode(item + stride) : cur;
+    // the next item's table entry: loaded now, stored to the other table in the last step
+    int n_arow = 0, n_orow = -1;
+    float n_sc = 1.0f;
+    if (has_next && tid < kBM) table_entry(nxt, n_arow, n_orow, n_sc);
 
     float16v acc[2][2];
 #pragma unroll
@@ -247,16 +288,6 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // In flight: the next step's activation chunks (one matrix phase ahead: they come from L2) and the raw
-    // weight bytes of the next two steps (the HBM-cold ones), in w[ks & 1].  The contraction has an even
-    // number of steps (whole superblocks), so the step pairs are unrolled and no register is copied.
-    // (The down launch, NM = 1, has no registers to spare for the second step and keeps one in flight.)
-    constexpr int kWDepth = NM == 2 ? 2 : 1;
-    u32x4 areg[8];
-    WRaw<QUANT> w[kWDepth];
-    load_step_w<QUANT>(0, wrow, du, w[0]);
-    load_step_a(0, arow_ptr, areg);
-    if constexpr (kWDepth == 2) load_step_w<QUANT>(1, wrow, du, w[kWDepth - 1]);
     auto step = [&](auto p_c, int ks) __attribute__((always_inline)) {
       constexpr int P = decltype(p_c)::value % kWDepth;
       __syncthreads();  // everyone has finished reading the previous step's tiles
@@ -272,11 +303,29 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
         if constexpr (QUANT == kQ6K) q6_unit_to_lds(w[P].u[i], du, &sB[rb * kLd]);
         else q8_unit_to_lds(w[P].u[i], &sB[rb * kLd + du * 32]);
       }
+      if (ks == nks - 1 && has_next && tid < kBM) {
+        // (the other table's last reader, the previous item's epilogue, finished before this item's first barrier)
+        sArow[(buf ^ 1) * kTable + tid] = n_arow;
+        sOrow[(buf ^ 1) * kTable + tid] = n_orow;
+        sScale[(buf ^ 1) * kTable + tid] = n_sc;
+      }
       XABE_MT(1);
       __syncthreads();
       XABE_MT(2);
-      if (ks + 1 < nks) load_step_a(ks + 1, arow_ptr, areg);  // in flight while the matrix cores work
-      if (ks + kWDepth < nks) load_step_w<QUANT>(ks + kWDepth, wrow, du, w[P]);
+      // loads of the coming steps, in flight while the matrix cores work; past the end of this item they
+      // are the first steps of the next one
+      if (ks + 1 < nks) {
+        load_step_a(ks + 1, arow_ptr, areg);
+      } else if (has_next) {
+        set_arow(buf ^ 1);
+        load_step_a(0, arow_ptr, areg);
+      }
+      if (ks + kWDepth < nks) {
+        load_step_w<QUANT>(ks + kWDepth, wrow, du, w[P]);
+      } else if (has_next) {
+        if (ks + kWDepth == nks) set_wrow(nxt);
+        load_step_w<QUANT>(ks + kWDepth - nks, wrow, du, w[P]);
+      }
       const _Float16* pa = &sA[(wm * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
       const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
       // Operand fragments one sub-step ahead, in two register sets: the four LDS reads of sub-step kk + 1 are
@@ -322,22 +371,25 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int r = wm * 64 + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-        const int orow = sOrow[r];
+        const int orow = sOrow[buf * kTable + r];
         if (orow < 0) continue;
         if (NM == 2) {
-          const int col = nt * 64 + wn * 32 + (lane & 31);
+          const int col = cur.nt * 64 + wn * 32 + (lane & 31);
           const float g = acc[mi][0][v] * kWScaleInv, u = acc[mi][1][v] * kWScaleInv;
           static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_f(g) * u);
         } else {
-          const float sc = sScale[r];
+          const float sc = sScale[buf * kTable + r];
 #pragma unroll
           for (int ni = 0; ni < 2; ++ni) {
-            const int col = nt * 128 + wn * 64 + ni * 32 + (lane & 31);
+            const int col = cur.nt * 128 + wn * 64 + ni * 32 + (lane & 31);
             static_cast<float*>(a.out)[(size_t)orow * a.n_rows + col] = sc * (acc[mi][ni][v] * kWScaleInv);
           }
         }
       }
     }
+    if (!has_next) break;
+    cur = nxt;
+    buf ^= 1;
   }
 }
 
@@ -411,7 +463,7 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
 template <int NM, bool ROUTED>
 static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
   const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * 2));
-  constexpr size_t smem = (size_t)(kBM + kBR) * kLd * sizeof(_Float16) + 3 * kBM * sizeof(int);
+  constexpr size_t smem = (size_t)(kBM + kBR) * kLd * sizeof(_Float16) + 2 * 3 * kBM * sizeof(int);
   auto kq6 = k_mfma_expert<kQ6K, NM, ROUTED>;
   auto kq8 = k_mfma_expert<kQ8_0, NM, ROUTED>;
   static bool configured = false;  // per instantiation; the attribute is per function, set once
