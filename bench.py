@@ -245,7 +245,9 @@ def main() -> int:
 MFMA_PEAK_TFLOPS = 2500.0
 # name -> (kind, tokens, layers rotated): the MoE block at other widths and the dense sibling
 OTHER_WORKLOADS = {"decode_b32": ("moe", 32, 16), "prefill_512": ("moe", 512, 4), "prefill_8192": ("moe", 8192, 2),
-                   "dense_b1": ("dense", 1, 4), "dense_b8": ("dense", 8, 4)}
+                   "dense_b1": ("dense", 1, 4), "dense_b8": ("dense", 8, 4),
+                   # the LM head (2048 -> 248 320, Q8_0: 540 MB per pass), two copies rotated
+                   "lm_head_b1": ("lm_head", 1, 2), "lm_head_b3": ("lm_head", 3, 2), "lm_head_b8": ("lm_head", 8, 2)}
 
 
 def other_workload(args) -> int:
@@ -259,6 +261,8 @@ def other_workload(args) -> int:
 
     torch.cuda.set_device(0)
     kind, T, L = OTHER_WORKLOADS[args.workload]
+    if kind == "lm_head":
+        return lm_head_workload(args, T, L)
     if kind == "moe":
         g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
         layers = [make_layer_device_only(X, g, seed=10_000 + 100 * l) for l in range(L)]
@@ -319,6 +323,68 @@ def other_workload(args) -> int:
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if kind == "moe" and T >= 64 else "f32",
         "data": "synthetic", "config": cfg, "roofline": roof, "algorithmic_bytes_per_step": byts, "flops_per_step": flops,
         "cpu_baseline": None}))
+    return 0
+
+
+def lm_head_workload(args, T, L) -> int:
+    """The LM-head GEMV over the real head's shape (Q8_0), logits for T tokens per step; HIP events on the
+    launch stream; the CPU leg is the oracle's sequential gemv over a slice of the vocabulary."""
+    import time
+
+    import numpy as np
+    import torch
+
+    import llmxabe_amd as X
+
+    torch.cuda.set_device(0)
+    g = X.LmHeadGeometry.qwen3_6(T)
+    heads = [X.HeadTensor.q8_0(X.synth_quant(X.ExpertQuant.Q8_0, 500 + l, g.elements(), 0.02)) for l in range(L)]
+    k = X.LmHeadKernels(g)
+    x = X.synth_normal_f32(99, T * g.hidden, 1.0).view(T, g.hidden)
+    logits = torch.zeros(T, g.vocab, device="cuda")
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    reps_w, reps = max(1, min(args.warmup, 32) // L), max(1, min(args.steps, 128) // L)
+    with torch.cuda.stream(stream):
+        for _ in range(reps_w):
+            for i in range(L):
+                k.forward(heads[i], x, T, logits)
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            for i in range(L):
+                k.forward(heads[i], x, T, logits)
+        e1.record(stream)
+        e1.synchronize()
+    steps = reps * L
+    ms = e0.elapsed_time(e1) / steps
+    byts = g.weight_bytes_read(T) + T * g.hidden * 4 + T * g.vocab * 4
+    gbps = byts / (ms * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+
+        rows = 16384
+        raw = heads[0].bytes[:rows * g.row_bytes()].cpu().numpy()
+        w = oracle.dequantize_row(1, raw)
+        xs = x.cpu().numpy()
+        t0, n = time.perf_counter(), 0
+        while time.perf_counter() - t0 < min(args.cpu_seconds, 10.0):
+            oracle.gemv(w, rows, g.hidden, xs[n % T])
+            n += 1
+        dt = time.perf_counter() - t0
+        cpu = {"value": n * rows / g.vocab / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+               "sample": f"sequential gemv over {rows} of the 248320 rows (dequantised beforehand), {n} token passes, scaled to the whole vocabulary"}
+    print(json.dumps({
+        "metric": "LM-head tokens/s at 1 GPU; HBM GB/s %peak", "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": steps, "warmup": reps_w * L, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": args.workload, "tokens": T, "hidden": g.hidden, "vocab": g.vocab, "format": "Q8_0",
+                   "weight_passes": g.weight_passes(T), "heads_rotated": L, "launch": "eager"},
+        "roofline": {"kernel": "k_lm_head_quant", "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": gbps / HBM_PEAK_GBPS, "traffic": None},
+        "algorithmic_bytes_per_step": byts, "cpu_baseline": cpu}))
     return 0
 
 

@@ -4,3 +4,4 @@ from .moe import (BLOCK_Q6_K_DEVICE_BYTES, BufferScope, ExpertQuant, LayerOpsKer
                   synth_normal_f32, synth_quant, to_device_layout)
 from .block import DEFAULT_RMS_EPS, DenseFfnBlock, DenseFfnLayerWeights, MoeBlock, MoeLayerWeights  # noqa: F401
 from .gguf import GgmlType, GgufError, GgufFile, TensorInfo, UploadedDenseFfnLayer, UploadedMoeLayer  # noqa: F401
+from .lm_head import ARGMAX_BLOCKS, MAX_BATCH_TILE, HeadFormat, HeadTensor, LmHeadGeometry, LmHeadKernels  # noqa: F401

@@ -11,7 +11,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libxabe_hip.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "xabe_hip.h")
 GGUF_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "xabe_gguf.h")
-HEADER_PATHS = (HEADER_PATH, GGUF_HEADER_PATH)
+LM_HEAD_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "xabe_lm_head.h")
+HEADER_PATHS = (HEADER_PATH, GGUF_HEADER_PATH, LM_HEAD_HEADER_PATH)
 
 sz = C.c_size_t
 vp = C.c_void_p
@@ -35,6 +36,10 @@ class MoeLayerWeightsC(C.Structure):
 
 class DenseLayerWeightsC(C.Structure):
     _fields_ = [("post_norm", vp), ("gate", QuantTensorC), ("up", QuantTensorC), ("down", QuantTensorC)]
+
+
+class LmHeadGeometryC(C.Structure):
+    _fields_ = [("hidden", sz), ("vocab", sz), ("max_tokens", sz)]
 
 
 class TensorInfoC(C.Structure):
@@ -159,6 +164,20 @@ _SIGNATURES = {
     "xabe_dense_ffn_layer_weights_of": (C.POINTER(DenseLayerWeightsC), [vp]),
     "xabe_dense_ffn_layer_quants": (C.c_int, [vp, C.POINTER(C.c_int * 3)]),
     "xabe_dense_ffn_layer_bytes": (sz, [vp]),
+    # include/xabe_lm_head.h
+    "xabe_head_format_from_ggml": (C.c_int, [C.c_int]),
+    "xabe_lm_head_geometry_qwen3_6": (LmHeadGeometryC, [sz]),
+    "xabe_lm_head_row_bytes_for": (sz, [C.POINTER(LmHeadGeometryC), C.c_int]),
+    "xabe_lm_head_weight_bytes_for": (sz, [C.POINTER(LmHeadGeometryC), C.c_int]),
+    "xabe_lm_head_elements": (sz, [C.POINTER(LmHeadGeometryC)]),
+    "xabe_lm_head_weight_passes": (sz, [C.POINTER(LmHeadGeometryC), sz]),
+    "xabe_lm_head_weight_bytes_read": (sz, [C.POINTER(LmHeadGeometryC), C.c_int, sz]),
+    "xabe_lm_head_new": (C.c_int, [C.POINTER(LmHeadGeometryC), C.POINTER(vp)]),
+    "xabe_lm_head_free": (None, [vp]),
+    "xabe_lm_head_geometry_of": (C.c_int, [vp, C.POINTER(LmHeadGeometryC)]),
+    "xabe_lm_head_forward": (C.c_int, [vp, vp, C.c_int, vp, sz, vp, sz, sz, vp, sz]),
+    "xabe_lm_head_argmax": (C.c_int, [vp, vp, vp, sz, sz, vp, sz, vp, sz, vp, sz]),
+    "xabe_lm_head_argmax_prob": (C.c_int, [vp, vp, vp, sz, sz, vp, sz]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
