@@ -1,0 +1,90 @@
+"""Every forward path is capturable into a hipGraph (no allocation, no host synchronisation, the live-token
+count read from device memory; crates/xabe-cuda/src/kernels/moe.rs:34-41, docs/TOOLCHAIN.md:107-142): a
+captured pass, replayed several times with eager work and synchronisations between the replays, gives the
+eager pass's bits every time."""
+import numpy as np
+import pytest
+
+from util import activations, make_layer
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def X():
+    import llmxabe_amd as X
+    return X
+
+
+def _replays(torch, stream, capture, outputs, scramble, eager_bits, what, rows=None):
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        capture()                      # warm-up on the capture stream: everything one-time happens here
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            capture()
+        for rep in range(4):
+            scramble()                 # eager work between replays: the outputs are overwritten
+            stream.synchronize()
+            graph.replay()
+            stream.synchronize()
+            for o, want in zip(outputs, eager_bits):
+                assert torch.equal(o.view(torch.int32)[:rows], want[:rows]), f"{what}: replay {rep} differs from the eager pass"
+
+
+@pytest.mark.parametrize("max_tokens,tokens", [(3, 3), (12, 9), (32, 32), (128, 100)])
+def test_moe_block_forward_replays(oracle, X, max_tokens, tokens):
+    import torch
+
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(max_tokens), max_tokens)
+    layer = make_layer(oracle, g, seed=8800 + max_tokens, router_q8=(max_tokens != 12),
+                       down_quant=X.ExpertQuant.Q8_0 if max_tokens == 12 else None)
+    blk = X.MoeBlock(g)
+    x = activations(8801, max_tokens, 2048, tokens)
+    ffn, lout = torch.zeros_like(x), torch.zeros_like(x)
+    blk.forward(layer.dev, x, tokens, ffn, lout)
+    torch.cuda.synchronize()
+    want = [ffn.view(torch.int32).clone(), lout.view(torch.int32).clone()]
+    stream = torch.cuda.Stream()
+
+    def scramble():
+        ffn.fill_(float("nan"))
+        lout.fill_(float("nan"))
+
+    _replays(torch, stream, lambda: blk.forward(layer.dev, x, tokens, ffn, lout), [ffn, lout], scramble, want,
+             f"block {max_tokens}/{tokens}", rows=tokens)   # rows past the live tokens are never written
+
+
+def test_dense_block_and_lm_head_replay(oracle, X):
+    import torch
+
+    H, I = 5120, 17408
+    q = X.ExpertQuant.Q6K
+    w = X.DenseFfnLayerWeights(1.0 + X.synth_normal_f32(44, H, 0.1), X.QuantTensor(X.synth_quant(q, 41, H * I, 0.02), q),
+                               X.QuantTensor(X.synth_quant(q, 42, H * I, 0.02), q), X.QuantTensor(X.synth_quant(q, 43, H * I, 0.02), q))
+    blk = X.DenseFfnBlock(H, I, 2)
+    x = X.synth_normal_f32(51, 2 * H, 1.0).view(2, H)
+    ffn, lout = torch.zeros_like(x), torch.zeros_like(x)
+    blk.forward(w, x, 2, ffn, lout)
+    torch.cuda.synchronize()
+    want = [ffn.view(torch.int32).clone(), lout.view(torch.int32).clone()]
+    stream = torch.cuda.Stream()
+    _replays(torch, stream, lambda: blk.forward(w, x, 2, ffn, lout), [ffn, lout],
+             lambda: (ffn.zero_(), lout.zero_()), want, "dense block")
+
+    g = X.LmHeadGeometry(2048, 8192, 3)
+    k = X.LmHeadKernels(g)
+    head = X.HeadTensor.q8_0(X.synth_quant(X.ExpertQuant.Q8_0, 61, g.elements(), 0.02))
+    hs = X.synth_normal_f32(62, 3 * 2048, 1.0).view(3, 2048)
+    logits = torch.zeros(3, g.vocab, device="cuda")
+    pv, pi = torch.zeros(512, device="cuda"), torch.zeros(512, dtype=torch.int32, device="cuda")
+    out = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    def head_pass():
+        k.forward(head, hs, 3, logits)
+        k.argmax(logits[2], g.vocab, pv, pi, out)
+
+    head_pass()
+    torch.cuda.synchronize()
+    want = [logits.view(torch.int32).clone(), out.clone()]
+    _replays(torch, stream, head_pass, [logits, out], lambda: (logits.fill_(-1.0), out.fill_(-5)), want, "LM head + argmax")
