@@ -35,7 +35,12 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kBM = 128;          // token rows per tile
 constexpr int kBR = 128;          // weight rows per tile
 constexpr int kBK = 128;          // contraction elements per step
-constexpr int kLd = kBK + 8;      // LDS row stride in halfs (272 B: 16-B reads are conflict-free)
+constexpr int kLd = kBK + 8;      // LDS row stride of the weight tile in halfs (272 B: 16-B reads are conflict-free)
+// The activation tile goes from global memory straight into LDS (global_load_lds_dwordx4: no registers, no
+// store instructions), which writes a wavefront's 64 pieces contiguously, so its rows are unpadded (256 B)
+// and the 16-byte chunks of a row are stored XOR-swizzled by the row number instead: chunk c of row r sits at
+// position c ^ (r & 15), and 16 consecutive rows reading the same chunk hit 16 different bank groups.
+constexpr int kLdA = kBK;
 constexpr float kWScale = 256.0f;
 constexpr float kWScaleInv = 1.0f / 256.0f;
 
@@ -108,17 +113,67 @@ __device__ __forceinline__ void q8_unit_to_lds(const Q8Raw& r, _Float16* bdst) {
     reinterpret_cast<u32x4*>(bdst)[w] = pack8(r.q[2 * w] ^ 0x80808080u, r.q[2 * w + 1] ^ 0x80808080u, off, s);
 }
 
+// Nothing moves across this point, in either direction, when the compiler schedules.
+__device__ __forceinline__ void order_fence() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// Raw blocks in flight.  The loads deliver the aligned dwords that cover each field; the funnel shifts that
+// turn them into the fields (q6_load / q8_load do both at once) are left to the step that consumes them: a
+// shift placed next to its load makes the wavefront wait for the data before it starts the matrix
+// instructions of the step in which the loads are only meant to be in flight.
+struct Q6Pend {
+  uint32_t qa[3], qb[3], qh[3], sc[3], dh, sh;
+};
+struct Q8Pend {
+  uint32_t e[9], dh, sh;
+};
+__device__ __forceinline__ void q6_issue(const uint8_t* base4, uint32_t lane_off, int half, int l8, Q6Pend& r) {
+  // every field of a unit starts a multiple of four bytes into the superblock: one shift serves all four
+  r.sh = (lane_off & 2u) << 3;
+  auto three = [&](uint32_t off, uint32_t (&d)[3]) __attribute__((always_inline)) {
+    const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + (off & ~3u));
+    d[0] = p[0], d[1] = p[1], d[2] = p[2];
+  };
+  three(lane_off + half * 64 + l8 * 8, r.qa);
+  three(lane_off + half * 64 + 32 + l8 * 8, r.qb);
+  three(lane_off + 128 + half * 32 + l8 * 8, r.qh);
+  {  // the scales are the last field but one of the block: the third dword only when the field spills into it
+    const uint32_t off = lane_off + 192 + half * 8;
+    const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + (off & ~3u));
+    r.sc[0] = p[0], r.sc[1] = p[1], r.sc[2] = p[r.sh ? 2 : 1];
+  }
+  r.dh = load_u16(base4, lane_off + 208);
+}
+__device__ __forceinline__ void q6_finish(const Q6Pend& p, Q6Raw& r) {
+  r.qa0 = __builtin_amdgcn_alignbit(p.qa[1], p.qa[0], p.sh), r.qa1 = __builtin_amdgcn_alignbit(p.qa[2], p.qa[1], p.sh);
+  r.qb0 = __builtin_amdgcn_alignbit(p.qb[1], p.qb[0], p.sh), r.qb1 = __builtin_amdgcn_alignbit(p.qb[2], p.qb[1], p.sh);
+  r.qh0 = __builtin_amdgcn_alignbit(p.qh[1], p.qh[0], p.sh), r.qh1 = __builtin_amdgcn_alignbit(p.qh[2], p.qh[1], p.sh);
+  r.sc0 = __builtin_amdgcn_alignbit(p.sc[1], p.sc[0], p.sh), r.sc1 = __builtin_amdgcn_alignbit(p.sc[2], p.sc[1], p.sh);
+  r.dh = p.dh;
+}
+__device__ __forceinline__ void q8_issue(const uint8_t* base4, uint32_t lane_off, Q8Pend& r) {
+  const uint32_t qoff = lane_off + 2;
+  r.sh = (qoff & 2u) << 3;
+  const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + (qoff & ~3u));
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r.e[i] = p[i];
+  r.e[8] = load_u16(base4, lane_off + (r.sh ? 32u : 0u));  // the block's last two codes (see q8_load)
+  r.dh = load_u16(base4, lane_off);
+}
+__device__ __forceinline__ void q8_finish(const Q8Pend& p, Q8Raw& r) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r.q[i] = __builtin_amdgcn_alignbit(p.e[i + 1], p.e[i], p.sh);
+  r.dh = p.dh;
+}
+
 template <int QUANT>
 struct WRaw {
-  typename std::conditional<QUANT == kQ6K, Q6Raw, Q8Raw>::type u[2];
+  typename std::conditional<QUANT == kQ6K, Q6Pend, Q8Pend>::type u[2];
 };
 
-// Global loads of one contraction step into registers: eight 16-byte activation chunks ...
-__device__ __forceinline__ void load_step_a(int ks, const _Float16* const (&arow_ptr)[8], u32x4 (&areg)[8]) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) areg[i] = *reinterpret_cast<const u32x4*>(arow_ptr[i] + (size_t)ks * kBK);
-}
-// ... and the raw blocks of this thread's two weight-row units.
+// Global loads of one contraction step into registers: the raw blocks of this thread's two weight-row units.
 template <int QUANT>
 __device__ __forceinline__ void load_unit_w(int ks, int i, const uint8_t* const (&wrow)[2], int du, WRaw<QUANT>& wreg) {
   {
@@ -126,11 +181,11 @@ __device__ __forceinline__ void load_unit_w(int ks, int i, const uint8_t* const 
       // step ks covers half (ks & 1) of superblock ks >> 1
       const uint8_t* p = wrow[i] + (size_t)(ks >> 1) * kQ6KBytes;
       const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
-      q6_load(p - mis, mis, ks & 1, du, wreg.u[i]);
+      q6_issue(p - mis, mis, ks & 1, du, wreg.u[i]);
     } else {
       const uint8_t* p = wrow[i] + (size_t)(ks * 4 + du) * kQ8Bytes;
       const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
-      q8_load(p - mis, mis, wreg.u[i]);
+      q8_issue(p - mis, mis, wreg.u[i]);
     }
   }
 }
@@ -154,10 +209,10 @@ static __device__ long long g_mfma_trace[512 * 32 * 4];
 
 template <int QUANT, int NM, bool ROUTED>
 __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
-  // 72.5 KB of LDS per workgroup (two per CU): dynamic, since the static limit is 64 KB
+  // 70.5 KB of LDS per workgroup (two per CU): dynamic, since the static limit is 64 KB
   extern __shared__ __attribute__((aligned(16))) uint8_t mfma_smem[];
   _Float16* sA = reinterpret_cast<_Float16*>(mfma_smem);
-  _Float16* sB = sA + kBM * kLd;
+  _Float16* sB = sA + kBM * kLdA;
   // row tables, two sets (this item's and the next one's), each kTable = 3 * kBM words apart
   constexpr int kTable = 3 * kBM;
   int* sArow = reinterpret_cast<int*>(sB + kBR * kLd);  // activation row index of each tile row
@@ -199,9 +254,10 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     const int mt = m_lo + item / n_ntiles;
     Item it{0, mt * kBM, min(kBM, valid - mt * kBM), item % n_ntiles};
     if (ROUTED) {
-      it.e = a.tile_list[4 + 4 * mt];
-      it.m0 = a.tile_list[4 + 4 * mt + 1];
-      it.rows = a.tile_list[4 + 4 * mt + 2];
+      // (scalars, read where decode is called: the steps' wait bookkeeping must not meet these loads later)
+      it.e = __builtin_amdgcn_readfirstlane(a.tile_list[4 + 4 * mt]);
+      it.m0 = __builtin_amdgcn_readfirstlane(a.tile_list[4 + 4 * mt + 1]);
+      it.rows = __builtin_amdgcn_readfirstlane(a.tile_list[4 + 4 * mt + 2]);
     }
     return it;
   };
@@ -219,20 +275,22 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       }
     }
   };
+  const ptrdiff_t up_minus_gate = NM == 2 ? a.w1 - a.w0 : 0;
   const uint8_t* wrow[2];        // weight rows this thread dequantises
-  const _Float16* arow_ptr[8];   // activation chunks this thread stages: 8 x 16 bytes per step
+  uint32_t arow_off[8];          // activation chunks this thread moves, 8 x 16 bytes per step: element offsets
   auto set_wrow = [&](const Item& it) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int rb = rb0 + 64 * i;
-      const uint8_t* base;
+      const uint8_t* base = a.w0;
       int wr;
       if (NM == 2) {
         const int half_n = rb >> 6, which = (rb >> 5) & 1, c = rb & 31;
-        base = which ? a.w1 : a.w0;
+        // (arithmetic, not a select of the two pointers: the compiler turns that into a per-lane load from the
+        // kernel arguments, a memory operation in the middle of the steps)
+        base += which ? up_minus_gate : (ptrdiff_t)0;
         wr = it.nt * 64 + half_n * 32 + c;
       } else {
-        base = a.w0;
         wr = it.nt * 128 + rb;
       }
       wrow[i] = base + (size_t)it.e * a.expert_bytes + (size_t)wr * row_bytes;
@@ -242,16 +300,31 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int c = tid + 256 * i;
-      arow_ptr[i] = a.a + (size_t)sArow[buf * kTable + (c >> 4)] * a.K + (c & 15) * 8;
+      // piece c of the tile lands at LDS byte 16 c: row c >> 4, position c & 15, which holds chunk pos ^ (row & 15)
+      const int row = c >> 4, chunk = (c & 15) ^ (row & 15);
+      arow_off[i] = (uint32_t)sArow[buf * kTable + row] * (uint32_t)a.K + (uint32_t)chunk * 8u;
     }
   };
 
-  // In flight per step: the next step's activation chunks (one matrix phase ahead: they come from L2) and the
-  // raw weight bytes of the next two steps (the HBM-cold ones), in w[ks & 1].  The contraction has an even
+  // this step's activation tile: eight 1 KB pieces per wavefront, global memory -> LDS
+  auto move_a = [&](int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const _Float16* src = a.a + ((size_t)arow_off[i] + (size_t)ks * kBK);
+      uint8_t* dst = reinterpret_cast<uint8_t*>(sA) + (256 * i + 64 * wave) * 16;  // + 16 * lane, by the hardware
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
+  };
+
+  // In flight per step: the raw weight bytes of the next two steps (the HBM-cold ones), in w[ks & 1]; the
+  // activation tile (L2-warm) is moved during the step's own write phase, behind the dequantisation.  The contraction has an even
   // number of steps (whole superblocks), so the step pairs are unrolled and no register is copied.
   // (The down launch, NM = 1, has no registers to spare for the second step and keeps one in flight.)
-  constexpr int kWDepth = NM == 2 ? 2 : 1;
-  u32x4 areg[8];
+  constexpr int kWDepth = 2;
+  // load instructions one step's two units issue at the very least: Q6_K ql lo, ql hi, qh, scales, d per unit;
+  // Q8_0 the codes (at most two 16-byte loads per unit could ever cover them... counted as one) and d
+  constexpr int kWLoadsAtLeast = QUANT == kQ6K ? 10 : 4;
   WRaw<QUANT> w[kWDepth];
 
   Item cur = decode(first);
@@ -268,13 +341,14 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     set_wrow(cur);
     set_arow(0);
     load_step_w<QUANT>(0, wrow, du, w[0]);
-    load_step_a(0, arow_ptr, areg);
     if constexpr (kWDepth == 2) load_step_w<QUANT>(1, wrow, du, w[kWDepth - 1]);
   }
   int buf = 0;
   for (int item = first;; item += stride) {
     const bool has_next = item + stride < local_total;
     const Item nxt = has_next ? decode(item + stride) : cur;
+    // (materialised here: a load sunk into the steps would put a full wait on one of their paths)
+    asm volatile("" ::"s"(nxt.e), "s"(nxt.m0), "s"(nxt.rows), "s"(nxt.nt));
     // the next item's table entry: loaded now, stored to the other table in the last step
     int n_arow = 0, n_orow = -1;
     float n_sc = 1.0f;
@@ -290,18 +364,25 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 
     auto step = [&](auto p_c, int ks) __attribute__((always_inline)) {
       constexpr int P = decltype(p_c)::value % kWDepth;
-      __syncthreads();  // everyone has finished reading the previous step's tiles
+      // first barrier of the step: everyone has finished reading the previous step's tiles (LDS reads only: the
+      // weight loads in flight stay in flight)
+      order_fence();
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      order_fence();
       XABE_MT(0);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int c = tid + 256 * i;
-        *reinterpret_cast<u32x4*>(&sA[(c >> 4) * kLd + (c & 15) * 8]) = areg[i];
-      }
+      move_a(ks);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int rb = rb0 + 64 * i;
-        if constexpr (QUANT == kQ6K) q6_unit_to_lds(w[P].u[i], du, &sB[rb * kLd]);
-        else q8_unit_to_lds(w[P].u[i], &sB[rb * kLd + du * 32]);
+        if constexpr (QUANT == kQ6K) {
+          Q6Raw r;
+          q6_finish(w[P].u[i], r);
+          q6_unit_to_lds(r, du, &sB[rb * kLd]);
+        } else {
+          Q8Raw r;
+          q8_finish(w[P].u[i], r);
+          q8_unit_to_lds(r, &sB[rb * kLd + du * 32]);
+        }
       }
       if (ks == nks - 1 && has_next && tid < kBM) {
         // (the other table's last reader, the previous item's epilogue, finished before this item's first barrier)
@@ -309,32 +390,35 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
         sOrow[(buf ^ 1) * kTable + tid] = n_orow;
         sScale[(buf ^ 1) * kTable + tid] = n_sc;
       }
+      // The raw weight bytes of the step after next (past the end of this item: the first steps of the next one),
+      // into the registers the dequantisation above has just released.  Issued after the activation pieces, so
+      // that the wait for those at the barrier leaves these in flight: they have two whole steps to arrive.
+      // (every step issues the same loads, so that the compiler's count of what is in flight is exact on every
+      // path: the last two steps of a workgroup's last item re-read two of its own steps and drop them)
+      const int ks_w = ks + kWDepth < nks ? ks + kWDepth : ks + kWDepth - nks;
+      if (ks + kWDepth == nks && has_next) set_wrow(nxt);
+      load_step_w<QUANT>(ks_w, wrow, du, w[P]);
       XABE_MT(1);
-      __syncthreads();
+      // Second barrier of the step, by hand: this wavefront's LDS stores and its activation pieces must have
+      // landed, the weight loads just issued need not.  Memory operations retire in order, so "all but the last
+      // kWLoadsAtLeast" covers the pieces; the count is a lower bound of the load instructions a step issues
+      // (one per field of each unit), so a miscount can only wait for more, never for less.
+      order_fence();
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kWLoadsAtLeast) : "memory");
+      order_fence();
       XABE_MT(2);
-      // loads of the coming steps, in flight while the matrix cores work; past the end of this item they
-      // are the first steps of the next one
-      if (ks + 1 < nks) {
-        load_step_a(ks + 1, arow_ptr, areg);
-      } else if (has_next) {
-        set_arow(buf ^ 1);
-        load_step_a(0, arow_ptr, areg);
-      }
-      if (ks + kWDepth < nks) {
-        load_step_w<QUANT>(ks + kWDepth, wrow, du, w[P]);
-      } else if (has_next) {
-        if (ks + kWDepth == nks) set_wrow(nxt);
-        load_step_w<QUANT>(ks + kWDepth - nks, wrow, du, w[P]);
-      }
-      const _Float16* pa = &sA[(wm * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
+      if (ks + 1 == nks && has_next) set_arow(buf ^ 1);
+      const _Float16* pa = &sA[(wm * 64 + (lane & 31)) * kLdA];
+      const int swz = lane & 15, khalf = lane >> 5;  // (the row's low four bits are the lane's)
       const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
       // Operand fragments one sub-step ahead, in two register sets: the four LDS reads of sub-step kk + 1 are
       // issued before the four matrix instructions of sub-step kk, so their latency hides behind 128 cycles of
       // matrix work instead of standing between every group of four.
       half8 fa[2][2], fb[2][2];
       auto frags = [&](int kk, int set) __attribute__((always_inline)) {
-        fa[set][0] = *reinterpret_cast<const half8*>(pa + kk * 16);
-        fa[set][1] = *reinterpret_cast<const half8*>(pa + 32 * kLd + kk * 16);
+        const int apos = ((kk * 2 + khalf) ^ swz) * 8;
+        fa[set][0] = *reinterpret_cast<const half8*>(pa + apos);
+        fa[set][1] = *reinterpret_cast<const half8*>(pa + 32 * kLdA + apos);
         fb[set][0] = *reinterpret_cast<const half8*>(pb + kk * 16);
         fb[set][1] = *reinterpret_cast<const half8*>(pb + 32 * kLd + kk * 16);
       };
@@ -463,7 +547,7 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
 template <int NM, bool ROUTED>
 static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
   const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * 2));
-  constexpr size_t smem = (size_t)(kBM + kBR) * kLd * sizeof(_Float16) + 2 * 3 * kBM * sizeof(int);
+  constexpr size_t smem = (size_t)(kBM * kLdA + kBR * kLd) * sizeof(_Float16) + 2 * 3 * kBM * sizeof(int);
   auto kq6 = k_mfma_expert<kQ6K, NM, ROUTED>;
   auto kq8 = k_mfma_expert<kQ8_0, NM, ROUTED>;
   static bool configured = false;  // per instantiation; the attribute is per function, set once
