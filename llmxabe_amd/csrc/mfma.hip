@@ -450,6 +450,8 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     }
 
     // epilogue.  acc[mi][ni][v]: tile row (v/4)*8 + (lane/32)*4 + v%4, tile column lane%32
+    // (transposing the tile through LDS so that every lane stores 16 bytes of a row was measured: two more
+    // barriers per item and the extra registers cost more than the 48 fewer store instructions gave)
 #pragma unroll
     for (int mi = 0; mi < 2; ++mi) {
 #pragma unroll
