@@ -32,7 +32,7 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kBM = 128;          // token rows per tile
+constexpr int kBM = 128;          // token rows per tile (64 in the narrow form: see k_mfma_expert's TBM)
 constexpr int kBR = 128;          // weight rows per tile
 constexpr int kBK = 128;          // contraction elements per step
 constexpr int kLd = kBK + 8;      // LDS row stride of the weight tile in halfs (272 B: 16-B reads are conflict-free)
@@ -207,23 +207,30 @@ static __device__ long long g_mfma_trace[512 * 32 * 4];
 #define XABE_MT(slot) do { } while (0)
 #endif
 
-template <int QUANT, int NM, bool ROUTED>
+// TBM: token rows per tile, 128 or 64.  The narrow form serves geometries whose experts see at most ~64 tokens
+// each (up to ~2000 tokens per pass): half the matrix instructions, activation bytes and output stores per
+// item, the same weight work.  A wavefront then owns 32 x 64 of the tile instead of 64 x 64; every output
+// element sees the same operands in the same order, so the two forms give the same bits.
+template <int QUANT, int NM, bool ROUTED, int TBM = 128>
 __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
+  static_assert(TBM == 128 || TBM == 64, "token tile");
+  constexpr int MI = TBM / 64;       // 32-row blocks of the tile per wavefront
+  constexpr int kAPieces = TBM / 16; // 16-byte activation pieces per thread and step
   // 70.5 KB of LDS per workgroup (two per CU): dynamic, since the static limit is 64 KB
   extern __shared__ __attribute__((aligned(16))) uint8_t mfma_smem[];
   _Float16* sA = reinterpret_cast<_Float16*>(mfma_smem);
-  _Float16* sB = sA + kBM * kLdA;
-  // row tables, two sets (this item's and the next one's), each kTable = 3 * kBM words apart
-  constexpr int kTable = 3 * kBM;
+  _Float16* sB = sA + TBM * kLdA;
+  // row tables, two sets (this item's and the next one's), each kTable = 3 * TBM words apart
+  constexpr int kTable = 3 * TBM;
   int* sArow = reinterpret_cast<int*>(sB + kBR * kLd);  // activation row index of each tile row
-  int* sOrow = sArow + kBM;                             // output row index, or -1 for a dead row
-  float* sScale = reinterpret_cast<float*>(sOrow + kBM);
+  int* sOrow = sArow + TBM;                             // output row index, or -1 for a dead row
+  float* sScale = reinterpret_cast<float*>(sOrow + TBM);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int valid = *a.valid_tokens;
   const int n_ntiles = a.n_rows / (NM == 2 ? 64 : 128);
-  const int n_mtiles = ROUTED ? a.tile_list[0] : (valid + kBM - 1) / kBM;
+  const int n_mtiles = ROUTED ? a.tile_list[0] : (valid + TBM - 1) / TBM;
   const int total = n_mtiles * n_ntiles;
   const int nks = a.K / kBK;
   const size_t row_bytes = QUANT == kQ6K ? (size_t)(a.K / 256) * kQ6KBytes : (size_t)(a.K / 32) * kQ8Bytes;
@@ -252,7 +259,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   struct Item { int e, m0, rows, nt; };
   auto decode = [&](int item) __attribute__((always_inline)) {
     const int mt = m_lo + item / n_ntiles;
-    Item it{0, mt * kBM, min(kBM, valid - mt * kBM), item % n_ntiles};
+    Item it{0, mt * TBM, min(TBM, valid - mt * TBM), item % n_ntiles};
     if (ROUTED) {
       // (scalars, read where decode is called: the steps' wait bookkeeping must not meet these loads later)
       it.e = __builtin_amdgcn_readfirstlane(a.tile_list[4 + 4 * mt]);
@@ -261,7 +268,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     }
     return it;
   };
-  // table entry of tile row `tid` (threads below kBM): activation row, output row (-1: dead), output scale
+  // table entry of tile row `tid` (threads below TBM): activation row, output row (-1: dead), output scale
   auto table_entry = [&](const Item& it, int& arow, int& orow, float& sc) __attribute__((always_inline)) {
     arow = 0, orow = -1, sc = 1.0f;
     if (tid < it.rows) {
@@ -277,7 +284,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   };
   const ptrdiff_t up_minus_gate = NM == 2 ? a.w1 - a.w0 : 0;
   const uint8_t* wrow[2];        // weight rows this thread dequantises
-  uint32_t arow_off[8];          // activation chunks this thread moves, 8 x 16 bytes per step: element offsets
+  uint32_t arow_off[kAPieces];   // activation chunks this thread moves, 16 bytes each per step: element offsets
   auto set_wrow = [&](const Item& it) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -298,7 +305,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   };
   auto set_arow = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kAPieces; ++i) {
       const int c = tid + 256 * i;
       // piece c of the tile lands at LDS byte 16 c: row c >> 4, position c & 15, which holds chunk pos ^ (row & 15)
       const int row = c >> 4, chunk = (c & 15) ^ (row & 15);
@@ -306,10 +313,10 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     }
   };
 
-  // this step's activation tile: eight 1 KB pieces per wavefront, global memory -> LDS
+  // this step's activation tile: 1 KB pieces (eight per wavefront for 128 rows), global memory -> LDS
   auto move_a = [&](int ks) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kAPieces; ++i) {
       const _Float16* src = a.a + ((size_t)arow_off[i] + (size_t)ks * kBK);
       uint8_t* dst = reinterpret_cast<uint8_t*>(sA) + (256 * i + 64 * wave) * 16;  // + 16 * lane, by the hardware
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
@@ -331,7 +338,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   {
     int arow, orow;
     float sc;
-    if (tid < kBM) {
+    if (tid < TBM) {
       table_entry(cur, arow, orow, sc);
       sArow[tid] = arow;
       sOrow[tid] = orow;
@@ -352,11 +359,11 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     // the next item's table entry: loaded now, stored to the other table in the last step
     int n_arow = 0, n_orow = -1;
     float n_sc = 1.0f;
-    if (has_next && tid < kBM) table_entry(nxt, n_arow, n_orow, n_sc);
+    if (has_next && tid < TBM) table_entry(nxt, n_arow, n_orow, n_sc);
 
-    float16v acc[2][2];
+    float16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -384,7 +391,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
           q8_unit_to_lds(r, &sB[rb * kLd + du * 32]);
         }
       }
-      if (ks == nks - 1 && has_next && tid < kBM) {
+      if (ks == nks - 1 && has_next && tid < TBM) {
         // (the other table's last reader, the previous item's epilogue, finished before this item's first barrier)
         sArow[(buf ^ 1) * kTable + tid] = n_arow;
         sOrow[(buf ^ 1) * kTable + tid] = n_orow;
@@ -408,17 +415,17 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       order_fence();
       XABE_MT(2);
       if (ks + 1 == nks && has_next) set_arow(buf ^ 1);
-      const _Float16* pa = &sA[(wm * 64 + (lane & 31)) * kLdA];
+      const _Float16* pa = &sA[(wm * (TBM / 2) + (lane & 31)) * kLdA];
       const int swz = lane & 15, khalf = lane >> 5;  // (the row's low four bits are the lane's)
       const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
       // Operand fragments one sub-step ahead, in two register sets: the four LDS reads of sub-step kk + 1 are
       // issued before the four matrix instructions of sub-step kk, so their latency hides behind 128 cycles of
       // matrix work instead of standing between every group of four.
-      half8 fa[2][2], fb[2][2];
+      half8 fa[2][MI], fb[2][2];
       auto frags = [&](int kk, int set) __attribute__((always_inline)) {
         const int apos = ((kk * 2 + khalf) ^ swz) * 8;
         fa[set][0] = *reinterpret_cast<const half8*>(pa + apos);
-        fa[set][1] = *reinterpret_cast<const half8*>(pa + 32 * kLdA + apos);
+        if constexpr (MI == 2) fa[set][MI - 1] = *reinterpret_cast<const half8*>(pa + 32 * kLdA + apos);
         fb[set][0] = *reinterpret_cast<const half8*>(pb + kk * 16);
         fb[set][1] = *reinterpret_cast<const half8*>(pb + 32 * kLd + kk * 16);
       };
@@ -430,8 +437,10 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][0], fb[c][0], acc[0][0], 0, 0, 0);
         acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][0], fb[c][1], acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][1], fb[c][0], acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][1], fb[c][1], acc[1][1], 0, 0, 0);
+        if constexpr (MI == 2) {
+          acc[MI - 1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][MI - 1], fb[c][0], acc[MI - 1][0], 0, 0, 0);
+          acc[MI - 1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][MI - 1], fb[c][1], acc[MI - 1][1], 0, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
       XABE_MT(3);
@@ -453,10 +462,10 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     // (transposing the tile through LDS so that every lane stores 16 bytes of a row was measured: two more
     // barriers per item and the extra registers cost more than the 48 fewer store instructions gave)
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
+    for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int r = wm * 64 + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+        const int r = wm * (TBM / 2) + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
         const int orow = sOrow[buf * kTable + r];
         if (orow < 0) continue;
         if (NM == 2) {
@@ -493,9 +502,9 @@ __global__ void __launch_bounds__(256) k_to_f16_rows(const float* __restrict__ x
   }
 }
 
-// Token-tile list: one entry per 128-slot chunk of each active expert's run.  One workgroup.
+// Token-tile list: one entry per `bm`-slot chunk of each active expert's run.  One workgroup.
 __global__ void __launch_bounds__(256) k_build_tiles(const int* __restrict__ expert_counts, int num_experts, int block_size,
-                                                      int capacity, int* __restrict__ tile_list) {
+                                                      int capacity, int bm, int* __restrict__ tile_list) {
   __shared__ int s_base[513], s_tiles[513];
   // exclusive prefixes, serially by one thread per array (num_experts <= 512)
   if (threadIdx.x == 0) {
@@ -509,7 +518,7 @@ __global__ void __launch_bounds__(256) k_build_tiles(const int* __restrict__ exp
     int acc = 0;
     for (int e = 0; e < num_experts; ++e) {
       s_tiles[e] = acc;
-      acc += (expert_counts[e] + kBM - 1) / kBM;
+      acc += (expert_counts[e] + bm - 1) / bm;
     }
     s_tiles[num_experts] = acc;
     tile_list[0] = min(acc, capacity);
@@ -517,13 +526,13 @@ __global__ void __launch_bounds__(256) k_build_tiles(const int* __restrict__ exp
   __syncthreads();
   for (int e = threadIdx.x; e < num_experts; e += 256) {
     const int c = expert_counts[e];
-    const int nt = (c + kBM - 1) / kBM;
+    const int nt = (c + bm - 1) / bm;
     for (int i = 0; i < nt; ++i) {
       const int idx = s_tiles[e] + i;
       if (idx >= capacity) break;
       tile_list[4 + 4 * idx + 0] = e;
-      tile_list[4 + 4 * idx + 1] = s_base[e] + i * kBM;
-      tile_list[4 + 4 * idx + 2] = min(kBM, c - i * kBM);
+      tile_list[4 + 4 * idx + 1] = s_base[e] + i * bm;
+      tile_list[4 + 4 * idx + 2] = min(bm, c - i * bm);
       tile_list[4 + 4 * idx + 3] = 0;
     }
   }
@@ -546,12 +555,20 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
   return true;
 }
 
-template <int NM, bool ROUTED>
+// Token-tile height for a geometry: the narrow tile while an expert's share of a full pass usually fits in it
+// (an average of 48 selections per expert; at 64 every second expert overflows into a second tile, measured
+// 702 against 695 us at 2048 tokens).
+static int routed_tile_rows(const xabe_moe_geometry& g) {
+  return g.max_tokens * g.experts_per_token <= 48 * g.num_experts ? 64 : kBM;
+}
+static int shared_tile_rows(const xabe_moe_geometry& g) { return g.max_tokens <= 64 ? 64 : kBM; }
+
+template <int NM, bool ROUTED, int TBM>
 static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
   const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * 2));
-  constexpr size_t smem = (size_t)(kBM * kLdA + kBR * kLd) * sizeof(_Float16) + 2 * 3 * kBM * sizeof(int);
-  auto kq6 = k_mfma_expert<kQ6K, NM, ROUTED>;
-  auto kq8 = k_mfma_expert<kQ8_0, NM, ROUTED>;
+  constexpr size_t smem = (size_t)(TBM * kLdA + kBR * kLd) * sizeof(_Float16) + 2 * 3 * TBM * sizeof(int);
+  auto kq6 = k_mfma_expert<kQ6K, NM, ROUTED, TBM>;
+  auto kq8 = k_mfma_expert<kQ8_0, NM, ROUTED, TBM>;
   static bool configured = false;  // per instantiation; the attribute is per function, set once
   if (!configured) {
     XABE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kq6), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -576,7 +593,8 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   const xabe_moe_geometry& g = k->g;
   XABE_TRY(to_f16(k, s, b, x));
   const int cap = (int)((b->n_tile_list - 4) / 4);
-  hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap,
+  const int bm = routed_tile_rows(g);
+  hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap, bm,
                      b->tile_list);
   XABE_HIP_TRY(hipGetLastError());
   MfmaArgs a;
@@ -595,7 +613,8 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   a.out = b->inter_h;
   a.K = (int)g.hidden;
   a.n_rows = (int)g.intermediate;
-  XABE_TRY((launch_mfma<2, true>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  if (bm == 64) XABE_TRY((launch_mfma<2, true, 64>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  else XABE_TRY((launch_mfma<2, true, 128>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
   // down -> partial[flat][H], scaled by the routing weight
   a.w0 = static_cast<const uint8_t*>(down.bytes);
   a.w1 = nullptr;
@@ -604,7 +623,8 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   a.out = b->partial;
   a.K = (int)g.intermediate;
   a.n_rows = (int)g.hidden;
-  XABE_TRY((launch_mfma<1, true>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
+  if (bm == 64) XABE_TRY((launch_mfma<1, true, 64>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
+  else XABE_TRY((launch_mfma<1, true, 128>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
   return XABE_OK;
 }
 
@@ -616,21 +636,24 @@ int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffer
   memset(&a, 0, sizeof(a));
   a.valid_tokens = b->valid_tokens;
   a.top_k = 1;
-  const size_t max_mtiles = (g.max_tokens + kBM - 1) / kBM;
+  const int bm = shared_tile_rows(g);
+  const size_t max_mtiles = (g.max_tokens + bm - 1) / bm;
   a.w0 = static_cast<const uint8_t*>(gate.bytes);
   a.w1 = static_cast<const uint8_t*>(up.bytes);
   a.a = reinterpret_cast<const _Float16*>(b->x_h);
   a.out = b->shared_inter_h;
   a.K = (int)g.hidden;
   a.n_rows = (int)g.intermediate;
-  XABE_TRY((launch_mfma<2, false>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  if (bm == 64) XABE_TRY((launch_mfma<2, false, 64>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  else XABE_TRY((launch_mfma<2, false, 128>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
   a.w0 = static_cast<const uint8_t*>(down.bytes);
   a.w1 = nullptr;
   a.a = reinterpret_cast<const _Float16*>(b->shared_inter_h);
   a.out = out;
   a.K = (int)g.intermediate;
   a.n_rows = (int)g.hidden;
-  XABE_TRY((launch_mfma<1, false>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
+  if (bm == 64) XABE_TRY((launch_mfma<1, false, 64>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
+  else XABE_TRY((launch_mfma<1, false, 128>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
   return XABE_OK;
 }
 
