@@ -506,22 +506,33 @@ __global__ void __launch_bounds__(256) k_to_f16_rows(const float* __restrict__ x
 __global__ void __launch_bounds__(256) k_build_tiles(const int* __restrict__ expert_counts, int num_experts, int block_size,
                                                       int capacity, int bm, int* __restrict__ tile_list) {
   __shared__ int s_base[513], s_tiles[513];
-  // exclusive prefixes, serially by one thread per array (num_experts <= 512)
-  if (threadIdx.x == 0) {
-    int acc = 0;
-    for (int e = 0; e < num_experts; ++e) {
-      s_base[e] = acc;
-      acc += (expert_counts[e] + block_size - 1) / block_size * block_size;
-    }
+  // exclusive prefixes of the padded run lengths and of the tile counts (num_experts <= 512): every thread
+  // takes two experts, the pair sums are scanned across the workgroup in nine doubling steps
+  __shared__ int s_scan[2][2][256];
+  const int t = threadIdx.x;
+  int pad[2], til[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int e = 2 * t + j;
+    const int c = e < num_experts ? expert_counts[e] : 0;
+    pad[j] = (c + block_size - 1) / block_size * block_size;
+    til[j] = (c + bm - 1) / bm;
   }
-  if (threadIdx.x == 64) {
-    int acc = 0;
-    for (int e = 0; e < num_experts; ++e) {
-      s_tiles[e] = acc;
-      acc += (expert_counts[e] + bm - 1) / bm;
-    }
-    s_tiles[num_experts] = acc;
-    tile_list[0] = min(acc, capacity);
+  s_scan[0][0][t] = pad[0] + pad[1];
+  s_scan[0][1][t] = til[0] + til[1];
+  __syncthreads();
+  int cur = 0;
+  for (int d = 1; d < 256; d <<= 1) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a) s_scan[cur ^ 1][a][t] = s_scan[cur][a][t] + (t >= d ? s_scan[cur][a][t - d] : 0);
+    cur ^= 1;
+    __syncthreads();
+  }
+  {
+    const int base = s_scan[cur][0][t] - (pad[0] + pad[1]), tiles = s_scan[cur][1][t] - (til[0] + til[1]);
+    if (2 * t < num_experts) s_base[2 * t] = base, s_tiles[2 * t] = tiles;
+    if (2 * t + 1 < num_experts) s_base[2 * t + 1] = base + pad[0], s_tiles[2 * t + 1] = tiles + til[0];
+    if (t == 255) tile_list[0] = min(s_scan[cur][1][t], capacity);
   }
   __syncthreads();
   for (int e = threadIdx.x; e < num_experts; e += 256) {
