@@ -119,14 +119,23 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
                                                           w->down_exps, w->shared_gate, w->shared_up, w->shared_down,
                                                           blk->normed, blk->n_act, blk->shexp, blk->n_act, &fused));
   if (!fused) {
-    XABE_TRY(xabe_moe_grouped_forward_partial(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps, w->down_exps,
-                                              blk->normed, blk->n_act));
-    if (wide && mfma_supported(blk->moe, blk->buffers, w->shared_gate.quant, w->shared_up.quant, w->shared_down.quant, false))
-      XABE_TRY(xabe_moe_shared_expert_mma(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
-                                          blk->normed, blk->n_act, blk->shexp, blk->n_act));
-    else
-      XABE_TRY(xabe_moe_shared_expert(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
-                                      blk->normed, blk->n_act, blk->shexp, blk->n_act));
+    const bool shared_mma =
+        wide && mfma_supported(blk->moe, blk->buffers, w->shared_gate.quant, w->shared_up.quant, w->shared_down.quant, false);
+    // the routed and the shared matrix-core paths read the same fp16 copy of the rows: made once here
+    if (shared_mma) {
+      XABE_TRY(mfma_convert_activations(blk->moe, as_stream(stream), blk->buffers, blk->normed));
+      blk->buffers->x_h_ready = true;
+    }
+    int st = xabe_moe_grouped_forward_partial(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps, w->down_exps,
+                                              blk->normed, blk->n_act);
+    if (st == XABE_OK && shared_mma)
+      st = xabe_moe_shared_expert_mma(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
+                                      blk->normed, blk->n_act, blk->shexp, blk->n_act);
+    else if (st == XABE_OK)
+      st = xabe_moe_shared_expert(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
+                                  blk->normed, blk->n_act, blk->shexp, blk->n_act);
+    blk->buffers->x_h_ready = false;
+    if (st != XABE_OK) return st;
   }
   // 5. routed sum, sigmoid gate, combine, residual
   return xabe_moe_gate_and_combine(blk->moe, stream, blk->buffers, w->shared_gate_inp, blk->normed, blk->shexp, residual,

@@ -75,6 +75,9 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
                                  xabe_quant_tensor up, xabe_quant_tensor down, const float* x);
 int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
                        xabe_quant_tensor up, xabe_quant_tensor down, const float* x, float* out);
+// fp16 copy of the activations both of the above start from; a caller that makes it once sets
+// `x_h_ready` on the buffers for the calls that follow and clears it afterwards
+int mfma_convert_activations(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, const float* x);
 
 }  // namespace xabe
 
@@ -109,6 +112,7 @@ struct xabe_moe_buffers {
   float* shared_inter;  // [token][intermediate]
   // matrix-core regime staging
   uint16_t* x_h;        // [token][hidden] fp16 activations
+  bool x_h_ready;       // the caller has converted this pass's activations already
   uint16_t* inter_h;    // [slot][intermediate] fp16
   uint16_t* shared_inter_h;
   int32_t* tile_list;   // device-built tile schedule

@@ -572,7 +572,11 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
 static int routed_tile_rows(const xabe_moe_geometry& g) {
   return g.max_tokens * g.experts_per_token <= 48 * g.num_experts ? 64 : kBM;
 }
-static int shared_tile_rows(const xabe_moe_geometry& g) { return g.max_tokens <= 64 ? 64 : kBM; }
+// The shared expert's launches are short of workgroups below a few thousand tokens: the narrow tile while all
+// of its items still start at once (two workgroups per compute unit), so that twice as many units share the work.
+static int shared_tile_rows(const xabe_moe_kernels* k, size_t row_tiles) {
+  return (k->g.max_tokens + 63) / 64 * row_tiles <= (size_t)k->num_cus * 2 ? 64 : kBM;
+}
 
 template <int NM, bool ROUTED, int TBM>
 static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
@@ -599,10 +603,14 @@ static int to_f16(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffe
   return XABE_OK;
 }
 
+int mfma_convert_activations(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, const float* x) {
+  return to_f16(k, s, b, x);
+}
+
 int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
                                  xabe_quant_tensor up, xabe_quant_tensor down, const float* x) {
   const xabe_moe_geometry& g = k->g;
-  XABE_TRY(to_f16(k, s, b, x));
+  if (!b->x_h_ready) XABE_TRY(to_f16(k, s, b, x));
   const int cap = (int)((b->n_tile_list - 4) / 4);
   const int bm = routed_tile_rows(g);
   hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap, bm,
@@ -642,29 +650,37 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
 int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
                        xabe_quant_tensor up, xabe_quant_tensor down, const float* x, float* out) {
   const xabe_moe_geometry& g = k->g;
-  XABE_TRY(to_f16(k, s, b, x));
+  if (!b->x_h_ready) XABE_TRY(to_f16(k, s, b, x));
   MfmaArgs a;
   memset(&a, 0, sizeof(a));
   a.valid_tokens = b->valid_tokens;
   a.top_k = 1;
-  const int bm = shared_tile_rows(g);
-  const size_t max_mtiles = (g.max_tokens + bm - 1) / bm;
   a.w0 = static_cast<const uint8_t*>(gate.bytes);
   a.w1 = static_cast<const uint8_t*>(up.bytes);
   a.a = reinterpret_cast<const _Float16*>(b->x_h);
   a.out = b->shared_inter_h;
   a.K = (int)g.hidden;
   a.n_rows = (int)g.intermediate;
-  if (bm == 64) XABE_TRY((launch_mfma<2, false, 64>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
-  else XABE_TRY((launch_mfma<2, false, 128>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  {
+    const size_t row_tiles = g.intermediate / 64;
+    const int bm = shared_tile_rows(k, row_tiles);
+    const size_t items = (g.max_tokens + bm - 1) / bm * row_tiles;
+    if (bm == 64) XABE_TRY((launch_mfma<2, false, 64>(k, gate.quant, a, items, s)));
+    else XABE_TRY((launch_mfma<2, false, 128>(k, gate.quant, a, items, s)));
+  }
   a.w0 = static_cast<const uint8_t*>(down.bytes);
   a.w1 = nullptr;
   a.a = reinterpret_cast<const _Float16*>(b->shared_inter_h);
   a.out = out;
   a.K = (int)g.intermediate;
   a.n_rows = (int)g.hidden;
-  if (bm == 64) XABE_TRY((launch_mfma<1, false, 64>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
-  else XABE_TRY((launch_mfma<1, false, 128>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
+  {
+    const size_t row_tiles = g.hidden / 128;
+    const int bm = shared_tile_rows(k, row_tiles);
+    const size_t items = (g.max_tokens + bm - 1) / bm * row_tiles;
+    if (bm == 64) XABE_TRY((launch_mfma<1, false, 64>(k, down.quant, a, items, s)));
+    else XABE_TRY((launch_mfma<1, false, 128>(k, down.quant, a, items, s)));
+  }
   return XABE_OK;
 }
 
