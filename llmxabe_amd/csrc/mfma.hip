@@ -313,14 +313,19 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     }
   };
 
-  // this step's activation tile: 1 KB pieces (eight per wavefront for 128 rows), global memory -> LDS
+  // this step's activation tile: 1 KB pieces (eight per wavefront for 128 rows), global memory -> LDS.
+  // Written as assembly on purpose: the compiler's wait bookkeeping treats the instruction as one that may
+  // complete out of order with everything else, and answers any later wait for a weight register with "wait
+  // for all of memory", which stalls every other step on the pieces it has just requested.  Unseen by that
+  // bookkeeping, the pieces are covered by the step's second barrier (written by hand below), and the waits
+  // the compiler computes for the weight registers only ever come out too strict, by the pieces it did not count.
+  const uint32_t lds_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)sA + (uint32_t)wave * 1024u;
   auto move_a = [&](int ks) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kAPieces; ++i) {
       const _Float16* src = a.a + ((size_t)arow_off[i] + (size_t)ks * kBK);
-      uint8_t* dst = reinterpret_cast<uint8_t*>(sA) + (256 * i + 64 * wave) * 16;  // + 16 * lane, by the hardware
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_a + 4096u * i);  // + 16 * lane, by the hardware
+      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(dst) : "memory", "m0");
     }
   };
 
@@ -329,9 +334,11 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   // number of steps (whole superblocks), so the step pairs are unrolled and no register is copied.
   // (The down launch, NM = 1, has no registers to spare for the second step and keeps one in flight.)
   constexpr int kWDepth = 2;
-  // load instructions one step's two units issue at the very least: Q6_K ql lo, ql hi, qh, scales, d per unit;
-  // Q8_0 the codes (at most two 16-byte loads per unit could ever cover them... counted as one) and d
-  constexpr int kWLoadsAtLeast = QUANT == kQ6K ? 10 : 4;
+  // load instructions one step's two units issue at the very least, one per separately addressed piece: Q6_K ql
+  // low, ql high, qh, the scales' first eight bytes, their conditional third dword, d; Q8_0 two 16-byte halves of
+  // the codes, the trailing two codes, d.  (No two of these are adjacent in memory or share an address the
+  // compiler could prove equal, so it cannot issue fewer; issuing more only makes the barrier's wait stricter.)
+  constexpr int kWLoadsAtLeast = QUANT == kQ6K ? 12 : 8;
   WRaw<QUANT> w[kWDepth];
 
   Item cur = decode(first);
@@ -347,8 +354,13 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     __syncthreads();
     set_wrow(cur);
     set_arow(0);
+    // (fenced apart: the waits the compiler places in the steps are the strictest any path into them needs, and
+    // with these two sets of loads interleaved here it would make every step wait for its newest loads)
+    order_fence();
     load_step_w<QUANT>(0, wrow, du, w[0]);
+    order_fence();
     if constexpr (kWDepth == 2) load_step_w<QUANT>(1, wrow, du, w[kWDepth - 1]);
+    order_fence();
   }
   int buf = 0;
   for (int item = first;; item += stride) {
