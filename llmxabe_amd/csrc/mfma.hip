@@ -473,19 +473,30 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     // epilogue.  acc[mi][ni][v]: tile row (v/4)*8 + (lane/32)*4 + v%4, tile column lane%32
     // (transposing the tile through LDS so that every lane stores 16 bytes of a row was measured: two more
     // barriers per item and the extra registers cost more than the 48 fewer store instructions gave)
+    // (the rows' table entries are all read first: one LDS round trip for the item instead of one per row)
+    int orows[MI][16];
+    [[maybe_unused]] float scs[MI][16];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int r = wm * (TBM / 2) + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-        const int orow = sOrow[buf * kTable + r];
+        orows[mi][v] = sOrow[buf * kTable + r];
+        if (NM == 1) scs[mi][v] = sScale[buf * kTable + r];
+      }
+    }
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int orow = orows[mi][v];
         if (orow < 0) continue;
         if (NM == 2) {
           const int col = cur.nt * 64 + wn * 32 + (lane & 31);
           const float g = acc[mi][0][v] * kWScaleInv, u = acc[mi][1][v] * kWScaleInv;
           static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_f(g) * u);
         } else {
-          const float sc = sScale[buf * kTable + r];
+          const float sc = scs[mi][v];
 #pragma unroll
           for (int ni = 0; ni < 2; ++ni) {
             const int col = cur.nt * 128 + wn * 64 + ni * 32 + (lane & 31);
