@@ -123,11 +123,16 @@ __device__ __forceinline__ void order_fence() {
 // turn them into the fields (q6_load / q8_load do both at once) are left to the step that consumes them: a
 // shift placed next to its load makes the wavefront wait for the data before it starts the matrix
 // instructions of the step in which the loads are only meant to be in flight.
+// (d stays the sixteen bits the load delivers until the step that consumes it widens them: widened here, the
+// compiler carries the narrow value across the item boundary and widens it right after an item's last step,
+// waiting there for the loads meant to be in flight under the epilogue)
 struct Q6Pend {
-  uint32_t qa[3], qb[3], qh[3], sc[3], dh, sh;
+  uint32_t qa[3], qb[3], qh[3], sc[3], sh;
+  uint16_t dh;
 };
 struct Q8Pend {
-  uint32_t e[9], dh, sh;
+  uint32_t e[8], sh;
+  uint16_t e8, dh;
 };
 __device__ __forceinline__ void q6_issue(const uint8_t* base4, uint32_t lane_off, int half, int l8, Q6Pend& r) {
   // every field of a unit starts a multiple of four bytes into the superblock: one shift serves all four
@@ -144,7 +149,7 @@ __device__ __forceinline__ void q6_issue(const uint8_t* base4, uint32_t lane_off
     const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + (off & ~3u));
     r.sc[0] = p[0], r.sc[1] = p[1], r.sc[2] = p[r.sh ? 2 : 1];
   }
-  r.dh = load_u16(base4, lane_off + 208);
+  r.dh = *reinterpret_cast<const uint16_t*>(base4 + lane_off + 208);
 }
 __device__ __forceinline__ void q6_finish(const Q6Pend& p, Q6Raw& r) {
   r.qa0 = __builtin_amdgcn_alignbit(p.qa[1], p.qa[0], p.sh), r.qa1 = __builtin_amdgcn_alignbit(p.qa[2], p.qa[1], p.sh);
@@ -159,12 +164,13 @@ __device__ __forceinline__ void q8_issue(const uint8_t* base4, uint32_t lane_off
   const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + (qoff & ~3u));
 #pragma unroll
   for (int i = 0; i < 8; ++i) r.e[i] = p[i];
-  r.e[8] = load_u16(base4, lane_off + (r.sh ? 32u : 0u));  // the block's last two codes (see q8_load)
-  r.dh = load_u16(base4, lane_off);
+  r.e8 = *reinterpret_cast<const uint16_t*>(base4 + lane_off + (r.sh ? 32u : 0u));  // the block's last two codes (see q8_load)
+  r.dh = *reinterpret_cast<const uint16_t*>(base4 + lane_off);
 }
 __device__ __forceinline__ void q8_finish(const Q8Pend& p, Q8Raw& r) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) r.q[i] = __builtin_amdgcn_alignbit(p.e[i + 1], p.e[i], p.sh);
+  for (int i = 0; i < 7; ++i) r.q[i] = __builtin_amdgcn_alignbit(p.e[i + 1], p.e[i], p.sh);
+  r.q[7] = __builtin_amdgcn_alignbit((uint32_t)p.e8, p.e[7], p.sh);
   r.dh = p.dh;
 }
 
@@ -261,22 +267,35 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     const int mt = m_lo + item / n_ntiles;
     Item it{0, mt * TBM, min(TBM, valid - mt * TBM), item % n_ntiles};
     if (ROUTED) {
-      // (scalars, read where decode is called: the steps' wait bookkeeping must not meet these loads later)
-      it.e = __builtin_amdgcn_readfirstlane(a.tile_list[4 + 4 * mt]);
-      it.m0 = __builtin_amdgcn_readfirstlane(a.tile_list[4 + 4 * mt + 1]);
-      it.rows = __builtin_amdgcn_readfirstlane(a.tile_list[4 + 4 * mt + 2]);
+      // The tile's entry through the scalar unit: a vector load here would be waited for with a count of zero,
+      // i.e. together with every store the previous item's epilogue has just issued.
+      typedef int int4v __attribute__((ext_vector_type(4)));
+      int4v ent;
+      const int* p = a.tile_list + 4 + 4 * mt;  // 16-byte aligned: the list starts on an allocation boundary
+      asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ent) : "s"(p));
+      it.e = ent.x;
+      it.m0 = ent.y;
+      it.rows = ent.z;
     }
     return it;
   };
-  // table entry of tile row `tid` (threads below TBM): activation row, output row (-1: dead), output scale
-  auto table_entry = [&](const Item& it, int& arow, int& orow, float& sc) __attribute__((always_inline)) {
-    arow = 0, orow = -1, sc = 1.0f;
+  // table entry of tile row `tid` (threads below TBM): activation row, output row (-1: dead), output scale.
+  // In two parts, so that nothing waits for a load it has just issued: the row's flat selection index is
+  // requested when the item is decoded, the entry is derived from it steps later.
+  auto table_flat = [&](const Item& it) __attribute__((always_inline)) {
+    // (an address that is always valid rather than a select on the loaded value, which would wait for it here)
+    return ROUTED ? a.sorted_token_ids[it.m0 + min(tid, it.rows - 1)] : 0;
+  };
+  auto table_scale = [&](const Item& it, int flat) __attribute__((always_inline)) {
+    return ROUTED && NM == 1 ? a.topk_weights[flat] : 1.0f;
+  };
+  auto table_entry = [&](const Item& it, int flat, int& arow, int& orow) __attribute__((always_inline)) {
+    arow = 0, orow = -1;
     if (tid < it.rows) {
       if (ROUTED) {
         const int slot = it.m0 + tid;
-        const int flat = a.sorted_token_ids[slot];
         if (NM == 2) { arow = flat / a.top_k; orow = slot; }
-        else { arow = slot; orow = flat; sc = a.topk_weights[flat]; }
+        else { arow = slot; orow = flat; }
       } else {
         arow = orow = it.m0 + tid;
       }
@@ -344,12 +363,12 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   Item cur = decode(first);
   {
     int arow, orow;
-    float sc;
     if (tid < TBM) {
-      table_entry(cur, arow, orow, sc);
+      const int flat = table_flat(cur);
+      table_entry(cur, flat, arow, orow);
       sArow[tid] = arow;
       sOrow[tid] = orow;
-      sScale[tid] = sc;
+      sScale[tid] = table_scale(cur, flat);
     }
     __syncthreads();
     set_wrow(cur);
@@ -363,15 +382,21 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     order_fence();
   }
   int buf = 0;
+  // (routed down launch: the output scales requested during the previous item, stored to this item's table at its
+  // start, by which time the load is many requests old and waiting for it waits for nothing else)
+  float carried_sc = 1.0f;
   for (int item = first;; item += stride) {
+    if constexpr (ROUTED && NM == 1) {
+      if (item != first && tid < TBM) sScale[buf * kTable + tid] = carried_sc;
+    }
     const bool has_next = item + stride < local_total;
     const Item nxt = has_next ? decode(item + stride) : cur;
     // (materialised here: a load sunk into the steps would put a full wait on one of their paths)
     asm volatile("" ::"s"(nxt.e), "s"(nxt.m0), "s"(nxt.rows), "s"(nxt.nt));
-    // the next item's table entry: loaded now, stored to the other table in the last step
-    int n_arow = 0, n_orow = -1;
-    float n_sc = 1.0f;
-    if (has_next && tid < TBM) table_entry(nxt, n_arow, n_orow, n_sc);
+    // the next item's table entries: the flat index requested now, the scale two steps before the end, both
+    // stored to the other table in the last step
+    int n_flat = 0;
+    if (has_next && tid < TBM) n_flat = table_flat(nxt);
 
     float16v acc[MI][2];
 #pragma unroll
@@ -389,6 +414,16 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       order_fence();
       XABE_MT(0);
+      if constexpr (ROUTED && NM == 1) {
+        // the next item's output scales, two steps before they are stored.  (First thing in the step: the
+        // compiler waits for everything in flight before it uses the flat index, and at this point that is the
+        // previous step's weight loads, a whole step old, and not yet this step's activation pieces.)
+        if (ks + kWDepth == nks && has_next && tid < TBM) {
+          int flat = n_flat;
+          asm volatile("" : "+v"(flat));
+          carried_sc = table_scale(nxt, flat);
+        }
+      }
       move_a(ks);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
@@ -405,9 +440,12 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       }
       if (ks == nks - 1 && has_next && tid < TBM) {
         // (the other table's last reader, the previous item's epilogue, finished before this item's first barrier)
+        int n_arow, n_orow, flat = n_flat;
+        asm volatile("" : "+v"(flat));  // (pins the entry's arithmetic here: hoisted to the item's start it would wait for the load there)
+        table_entry(nxt, flat, n_arow, n_orow);
         sArow[(buf ^ 1) * kTable + tid] = n_arow;
         sOrow[(buf ^ 1) * kTable + tid] = n_orow;
-        sScale[(buf ^ 1) * kTable + tid] = n_sc;
+        if constexpr (!(ROUTED && NM == 1)) sScale[(buf ^ 1) * kTable + tid] = 1.0f;
       }
       // The raw weight bytes of the step after next (past the end of this item: the first steps of the next one),
       // into the registers the dequantisation above has just released.  Issued after the activation pieces, so
@@ -461,10 +499,14 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 #endif
     };
     if constexpr (kWDepth == 2) {
-      for (int ks = 0; ks < nks; ks += 2) {
+      // (at least one pair of steps, and written so: a path around the loop would count for the compiler's waits
+      // after it, and on that path the loads issued just before the loop are the newest)
+      int ks = 0;
+      do {
         step(std::integral_constant<int, 0>{}, ks);
         step(std::integral_constant<int, 1>{}, ks + 1);
-      }
+        ks += 2;
+      } while (ks < nks);
     } else {
 #pragma unroll 1
       for (int ks = 0; ks < nks; ++ks) step(std::integral_constant<int, 0>{}, ks);
