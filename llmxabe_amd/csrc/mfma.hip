@@ -119,58 +119,49 @@ __device__ __forceinline__ void order_fence() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-// Raw blocks in flight.  The loads deliver the aligned dwords that cover each field; the funnel shifts that
-// turn them into the fields (q6_load / q8_load do both at once) are left to the step that consumes them: a
-// shift placed next to its load makes the wavefront wait for the data before it starts the matrix
-// instructions of the step in which the loads are only meant to be in flight.
+// Raw blocks in flight, in the registers the loads deliver them to.  Blocks sit at two-byte alignment (210- and
+// 34-byte blocks) and the fields are read where they lie: vector memory loads on this hardware take any
+// alignment, which is what the compiler itself relies on for a memcpy from a byte pointer.
 // (d stays the sixteen bits the load delivers until the step that consumes it widens them: widened here, the
 // compiler carries the narrow value across the item boundary and widens it right after an item's last step,
 // waiting there for the loads meant to be in flight under the epilogue)
 struct Q6Pend {
-  uint32_t qa[3], qb[3], qh[3], sc[3], sh;
+  uint2 qa, qb, qh, sc;
   uint16_t dh;
 };
 struct Q8Pend {
-  uint32_t e[8], sh;
-  uint16_t e8, dh;
+  u32x4 lo, hi;
+  uint16_t dh;
 };
-__device__ __forceinline__ void q6_issue(const uint8_t* base4, uint32_t lane_off, int half, int l8, Q6Pend& r) {
-  // every field of a unit starts a multiple of four bytes into the superblock: one shift serves all four
-  r.sh = (lane_off & 2u) << 3;
-  auto three = [&](uint32_t off, uint32_t (&d)[3]) __attribute__((always_inline)) {
-    const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + (off & ~3u));
-    d[0] = p[0], d[1] = p[1], d[2] = p[2];
-  };
-  three(lane_off + half * 64 + l8 * 8, r.qa);
-  three(lane_off + half * 64 + 32 + l8 * 8, r.qb);
-  three(lane_off + 128 + half * 32 + l8 * 8, r.qh);
-  {  // the scales are the last field but one of the block: the third dword only when the field spills into it
-    const uint32_t off = lane_off + 192 + half * 8;
-    const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + (off & ~3u));
-    r.sc[0] = p[0], r.sc[1] = p[1], r.sc[2] = p[r.sh ? 2 : 1];
-  }
-  r.dh = *reinterpret_cast<const uint16_t*>(base4 + lane_off + 208);
+template <typename T>
+__device__ __forceinline__ T load_any(const uint8_t* p) {
+  T v;
+  __builtin_memcpy(&v, p, sizeof(T));
+  return v;
+}
+// unit l8 of half `half` of the superblock at `blk` (field offsets: crates/xabe-kernels/src/quant.rs:725-729)
+__device__ __forceinline__ void q6_issue(const uint8_t* blk, int half, int l8, Q6Pend& r) {
+  r.qa = load_any<uint2>(blk + half * 64 + l8 * 8);
+  r.qb = load_any<uint2>(blk + half * 64 + 32 + l8 * 8);
+  r.qh = load_any<uint2>(blk + 128 + half * 32 + l8 * 8);
+  r.sc = load_any<uint2>(blk + 192 + half * 8);
+  r.dh = load_any<uint16_t>(blk + 208);
 }
 __device__ __forceinline__ void q6_finish(const Q6Pend& p, Q6Raw& r) {
-  r.qa0 = __builtin_amdgcn_alignbit(p.qa[1], p.qa[0], p.sh), r.qa1 = __builtin_amdgcn_alignbit(p.qa[2], p.qa[1], p.sh);
-  r.qb0 = __builtin_amdgcn_alignbit(p.qb[1], p.qb[0], p.sh), r.qb1 = __builtin_amdgcn_alignbit(p.qb[2], p.qb[1], p.sh);
-  r.qh0 = __builtin_amdgcn_alignbit(p.qh[1], p.qh[0], p.sh), r.qh1 = __builtin_amdgcn_alignbit(p.qh[2], p.qh[1], p.sh);
-  r.sc0 = __builtin_amdgcn_alignbit(p.sc[1], p.sc[0], p.sh), r.sc1 = __builtin_amdgcn_alignbit(p.sc[2], p.sc[1], p.sh);
+  r.qa0 = p.qa.x, r.qa1 = p.qa.y;
+  r.qb0 = p.qb.x, r.qb1 = p.qb.y;
+  r.qh0 = p.qh.x, r.qh1 = p.qh.y;
+  r.sc0 = p.sc.x, r.sc1 = p.sc.y;
   r.dh = p.dh;
 }
-__device__ __forceinline__ void q8_issue(const uint8_t* base4, uint32_t lane_off, Q8Pend& r) {
-  const uint32_t qoff = lane_off + 2;
-  r.sh = (qoff & 2u) << 3;
-  const uint32_t* p = reinterpret_cast<const uint32_t*>(base4 + (qoff & ~3u));
-#pragma unroll
-  for (int i = 0; i < 8; ++i) r.e[i] = p[i];
-  r.e8 = *reinterpret_cast<const uint16_t*>(base4 + lane_off + (r.sh ? 32u : 0u));  // the block's last two codes (see q8_load)
-  r.dh = *reinterpret_cast<const uint16_t*>(base4 + lane_off);
+__device__ __forceinline__ void q8_issue(const uint8_t* blk, Q8Pend& r) {
+  r.dh = load_any<uint16_t>(blk);
+  r.lo = load_any<u32x4>(blk + 2);
+  r.hi = load_any<u32x4>(blk + 18);
 }
 __device__ __forceinline__ void q8_finish(const Q8Pend& p, Q8Raw& r) {
 #pragma unroll
-  for (int i = 0; i < 7; ++i) r.q[i] = __builtin_amdgcn_alignbit(p.e[i + 1], p.e[i], p.sh);
-  r.q[7] = __builtin_amdgcn_alignbit((uint32_t)p.e8, p.e[7], p.sh);
+  for (int i = 0; i < 4; ++i) r.q[i] = p.lo[i], r.q[4 + i] = p.hi[i];
   r.dh = p.dh;
 }
 
@@ -185,13 +176,9 @@ __device__ __forceinline__ void load_unit_w(int ks, int i, const uint8_t* const 
   {
     if constexpr (QUANT == kQ6K) {
       // step ks covers half (ks & 1) of superblock ks >> 1
-      const uint8_t* p = wrow[i] + (size_t)(ks >> 1) * kQ6KBytes;
-      const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
-      q6_issue(p - mis, mis, ks & 1, du, wreg.u[i]);
+      q6_issue(wrow[i] + (size_t)(ks >> 1) * kQ6KBytes, ks & 1, du, wreg.u[i]);
     } else {
-      const uint8_t* p = wrow[i] + (size_t)(ks * 4 + du) * kQ8Bytes;
-      const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
-      q8_issue(p - mis, mis, wreg.u[i]);
+      q8_issue(wrow[i] + (size_t)(ks * 4 + du) * kQ8Bytes, wreg.u[i]);
     }
   }
 }
@@ -354,10 +341,10 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   // (The down launch, NM = 1, has no registers to spare for the second step and keeps one in flight.)
   constexpr int kWDepth = 2;
   // load instructions one step's two units issue at the very least, one per separately addressed piece: Q6_K ql
-  // low, ql high, qh, the scales' first eight bytes, their conditional third dword, d; Q8_0 two 16-byte halves of
-  // the codes, the trailing two codes, d.  (No two of these are adjacent in memory or share an address the
-  // compiler could prove equal, so it cannot issue fewer; issuing more only makes the barrier's wait stricter.)
-  constexpr int kWLoadsAtLeast = QUANT == kQ6K ? 12 : 8;
+  // low, ql high, qh, scales, d; Q8_0 the two 16-byte halves of the codes and d.  (No two pieces of a unit
+  // are adjacent in memory except the scales and d, ten bytes that no single load covers, so the compiler cannot
+  // issue fewer; issuing more only makes the barrier's wait stricter.)
+  constexpr int kWLoadsAtLeast = QUANT == kQ6K ? 10 : 6;
   WRaw<QUANT> w[kWDepth];
 
   Item cur = decode(first);
