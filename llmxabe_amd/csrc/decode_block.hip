@@ -108,8 +108,8 @@ __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, cons
   for (int t = 0; t < TC; ++t) lane_x_load<QUANT>(xrow[t], koff, g, x[t]);
   lane_x_load<QUANT>(norm_w, koff, g, nw);
   Raw r[NM];
-  load_raw<QUANT>(w0 + (size_t)row0 * row_bytes, true, g, r[0]);
-  if constexpr (NM == 2) load_raw<QUANT>(w1 + (size_t)row0 * row_bytes, true, g, r[NM - 1]);
+  load_raw<QUANT, true>(w0 + (size_t)row0 * row_bytes, true, g, r[0]);
+  if constexpr (NM == 2) load_raw<QUANT, true>(w1 + (size_t)row0 * row_bytes, true, g, r[NM - 1]);
 #pragma unroll
   for (int t = 0; t < TC; ++t) {
     float s = 0.0f;
@@ -284,8 +284,8 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
       for (int d = 0; d < DEPTH; ++d) {
         if (d < d0 || d >= d1) continue;
         const int row0 = wave_row0 + d * RPS;  // the tiles divide the rows exactly (checked by the host)
-        load_raw<RQ>(wg + (size_t)row0 * row_bytes, true, g, r[d][0]);
-        load_raw<RQ>(wu + (size_t)row0 * row_bytes, true, g, r[d][1]);
+        load_raw<RQ, true>(wg + (size_t)row0 * row_bytes, true, g, r[d][0]);
+        load_raw<RQ, true>(wu + (size_t)row0 * row_bytes, true, g, r[d][1]);
       }
     };
     // The routing wavefront finishes the softmax before it requests its own rows: its neighbours' requests
@@ -371,7 +371,7 @@ __global__ void __launch_bounds__(256) k_decode_down(DecodeArgs a) {
   const size_t rb_s = (size_t)(a.I / Fmt<SQ>::kBlockElems) * Fmt<SQ>::kBlockBytes;
   const size_t rb_r = (size_t)(a.I / Fmt<RQ>::kBlockElems) * Fmt<RQ>::kBlockBytes;
   RawS rs;
-  load_raw<SQ>(a.sdown + (size_t)row0 * rb_s, true, gs, rs);
+  load_raw<SQ, true>(a.sdown + (size_t)row0 * rb_s, true, gs, rs);
   if (t >= valid) return;
   // round two: the selected experts' rows
   RawR rr[kMaxTopK];
@@ -380,7 +380,7 @@ __global__ void __launch_bounds__(256) k_decode_down(DecodeArgs a) {
     const int e = min(max(__builtin_amdgcn_readlane(my_e, k), 0), a.E - 1);
     // k >= top_k reads expert 0's rows and never uses them: an unconditional load keeps all of round two
     // in one basic block, so every load is issued before the first wait
-    load_raw<RQ>(a.down + (size_t)e * a.down_bytes + (size_t)row0 * rb_r, true, gr, rr[k]);
+    load_raw<RQ, true>(a.down + (size_t)e * a.down_bytes + (size_t)row0 * rb_r, true, gr, rr[k]);
   }
   // the activation rows arrived before the weights (loads return in order); publish them to LDS
 #pragma unroll

@@ -163,7 +163,8 @@ __device__ __forceinline__ void raw_zero<kF32>(F32Raw& r) {
 }
 
 // Loads this lane's block of the step that starts at `chunk` (any 2-byte alignment).
-template <int QUANT>
+// DIRECT: Q6_K fields read at their own alignment (q6_load_direct); the Raw is the same.
+template <int QUANT, bool DIRECT = false>
 __device__ __forceinline__ void load_raw(const uint8_t* chunk, bool active, const LaneGeom& g,
                                          typename Fmt<QUANT>::Raw& r) {
   if (!active) {
@@ -172,7 +173,8 @@ __device__ __forceinline__ void load_raw(const uint8_t* chunk, bool active, cons
   }
   const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(chunk) & 3u);
   const uint8_t* chunk4 = chunk - mis;
-  if constexpr (QUANT == kQ6K) q6_load(chunk4, g.lane_off + mis, g.half, g.l8, r);
+  if constexpr (QUANT == kQ6K && DIRECT) q6_load_direct(chunk4, g.lane_off + mis, g.half, g.l8, r);
+  else if constexpr (QUANT == kQ6K) q6_load(chunk4, g.lane_off + mis, g.half, g.l8, r);
   else if constexpr (QUANT == kQ8_0) q8_load(chunk4, g.lane_off + mis, r);
   else f32_load(chunk, g.lane_off, r);
 }

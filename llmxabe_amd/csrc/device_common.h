@@ -185,6 +185,24 @@ __device__ __forceinline__ void q6_load(const uint8_t* chunk4, uint32_t lane_off
   load8_funnel_tail(chunk4, lane_off + 192 + half * 8, r.sc0, r.sc1);
   r.dh = load_u16(chunk4, lane_off + 208);
 }
+// The same fields read where they lie, at the block's own two-byte alignment (vector memory loads take any
+// alignment): the same Raw, with four load instructions of eight bytes instead of eleven dwords and no shifts.
+// Slower than the aligned windows where a wavefront streams long runs of consecutive blocks (dispatch-table
+// and long-row kernels: 202 against 211 us per block at 32 tokens), faster where it reads a few short rows
+// per request (the decode block's launches: 37.1 against 36.0 us per block at 3 tokens).
+__device__ __forceinline__ void q6_load_direct(const uint8_t* chunk4, uint32_t lane_off, int half, int l8, Q6Raw& r) {
+  const uint8_t* blk = chunk4 + lane_off;
+  uint2 v;
+  __builtin_memcpy(&v, blk + half * 64 + l8 * 8, 8);
+  r.qa0 = v.x, r.qa1 = v.y;
+  __builtin_memcpy(&v, blk + half * 64 + 32 + l8 * 8, 8);
+  r.qb0 = v.x, r.qb1 = v.y;
+  __builtin_memcpy(&v, blk + 128 + half * 32 + l8 * 8, 8);
+  r.qh0 = v.x, r.qh1 = v.y;
+  __builtin_memcpy(&v, blk + 192 + half * 8, 8);
+  r.sc0 = v.x, r.sc1 = v.y;
+  r.dh = load_u16(chunk4, lane_off + 208);
+}
 
 __device__ __forceinline__ float ub0(uint32_t v) { return (float)(v & 0xffu); }
 __device__ __forceinline__ float ub1(uint32_t v) { return (float)((v >> 8) & 0xffu); }

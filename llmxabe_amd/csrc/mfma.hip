@@ -331,7 +331,12 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     for (int i = 0; i < kAPieces; ++i) {
       const _Float16* src = a.a + ((size_t)arow_off[i] + (size_t)ks * kBK);
       const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_a + 4096u * i);  // + 16 * lane, by the hardware
+      // (m0 is named as clobbered so that the compiler sets it again before any use of its own; it warns that it
+      // does not preserve the register across the statement, which is what is wanted here)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
       asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(dst) : "memory", "m0");
+#pragma clang diagnostic pop
     }
   };
 
