@@ -637,7 +637,9 @@ static int shared_tile_rows(const xabe_moe_kernels* k, size_t row_tiles) {
 
 template <int NM, bool ROUTED, int TBM>
 static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
-  const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * 2));
+  // workgroups resident per CU: the narrow tile's registers (about 150) and LDS (51.5 KB) leave room for a third
+  const size_t per_cu = TBM == 64 ? 3 : 2;
+  const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * per_cu));
   constexpr size_t smem = (size_t)(TBM * kLdA + kBR * kLd) * sizeof(_Float16) + 2 * 3 * TBM * sizeof(int);
   auto kq6 = k_mfma_expert<kQ6K, NM, ROUTED, TBM>;
   auto kq8 = k_mfma_expert<kQ8_0, NM, ROUTED, TBM>;
