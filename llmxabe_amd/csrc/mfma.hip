@@ -506,7 +506,10 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
 
     // epilogue.  acc[mi][ni][v]: tile row (v/4)*8 + (lane/32)*4 + v%4, tile column lane%32
     // (transposing the tile through LDS so that every lane stores 16 bytes of a row was measured: two more
-    // barriers per item and the extra registers cost more than the 48 fewer store instructions gave)
+    // barriers per item and the extra registers cost more than the 48 fewer store instructions gave; so was
+    // the transposed product, weights as the first operand, whose lanes hold four consecutive columns of one
+    // token row: a quarter of the store instructions, but each touches 32 rows' cache lines with 32 bytes
+    // instead of two rows' with 128, and the block took 1365 against 1333 us at 8192 tokens)
     // (the rows' table entries are all read first: one LDS round trip for the item instead of one per row)
     int orows[MI][16];
     [[maybe_unused]] float scs[MI][16];
