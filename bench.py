@@ -245,7 +245,7 @@ def main() -> int:
 MFMA_PEAK_TFLOPS = 2500.0
 # name -> (kind, tokens, layers rotated): the MoE block at other widths and the dense sibling
 OTHER_WORKLOADS = {"decode_b32": ("moe", 32, 16), "prefill_512": ("moe", 512, 4), "prefill_8192": ("moe", 8192, 2),
-                   "dense_b1": ("dense", 1, 4), "dense_b8": ("dense", 8, 4),
+                   "dense_b1": ("dense", 1, 4), "dense_b8": ("dense", 8, 4), "dense_2048": ("dense", 2048, 2),
                    # the LM head (2048 -> 248 320, Q8_0: 540 MB per pass), two copies rotated
                    "lm_head_b1": ("lm_head", 1, 2), "lm_head_b3": ("lm_head", 3, 2), "lm_head_b8": ("lm_head", 8, 2)}
 
@@ -312,7 +312,7 @@ def other_workload(args) -> int:
         cfg = {"workload": "dense_ffn_" + args.workload, "tokens": T, "hidden": 5120, "intermediate": 17408,
                "quant": "Q6_K", "layers_rotated": L, "launch": "eager"}
     gbps, tflops = byts / (ms * 1e-3) / 1e9, flops / (ms * 1e-3) / 1e12
-    mfma_bound = args.workload == "prefill_8192"
+    mfma_bound = args.workload in ("prefill_8192", "dense_2048")
     roof = ({"kernel": "whole block", "bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
              "frac": tflops / MFMA_PEAK_TFLOPS, "traffic": None} if mfma_bound else
             {"kernel": "whole block", "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -320,7 +320,7 @@ def other_workload(args) -> int:
     print(json.dumps({
         "metric": "MoE-block tokens/s at 1 GPU; decode HBM GB/s %peak; prefill MFMA util %", "value": T / (ms * 1e-3),
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": reps_w * L, "ms_per_step": ms, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if kind == "moe" and T >= 64 else "f32",
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if T >= 64 else "f32",
         "data": "synthetic", "config": cfg, "roofline": roof, "algorithmic_bytes_per_step": byts, "flops_per_step": flops,
         "cpu_baseline": None}))
     return 0
