@@ -107,7 +107,10 @@ size_t xabe_expert_quant_file_block_bytes(int quant); /* M:366-374 */
 size_t xabe_expert_quant_block_bytes(int quant);
 int xabe_expert_quant_is_community(int quant);        /* M:348-350 */
 
-/* A quantized stack resident on the device.  `bytes` is a device pointer to `len` bytes. */
+/* A quantized stack resident on the device.  `bytes` is a device pointer to `len` bytes and must lie on a
+ * 16-byte boundary (any device allocation does; a sub-tensor of one must be placed accordingly): every entry
+ * point that takes a stack answers XABE_ERR_INVALID_ARGUMENT otherwise.  Inside the stack, blocks sit wherever
+ * their 210- or 34-byte stride puts them. */
 typedef struct xabe_quant_tensor {
   const void* bytes;
   size_t len;

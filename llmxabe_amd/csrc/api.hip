@@ -683,6 +683,16 @@ static int check_shared_stacks(const xabe_moe_kernels* k, xabe_quant_tensor gate
   return XABE_OK;
 }
 
+int xabe::check_layer_stacks(const xabe_moe_kernels* k, const xabe_moe_layer_weights* w) {
+  XABE_TRY(check_routed_stacks(k, w->gate_exps, w->up_exps, w->down_exps));
+  XABE_TRY(check_shared_stacks(k, w->shared_gate, w->shared_up, w->shared_down));
+  if (!w->router || !w->post_norm || !w->shared_gate_inp)
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "layer weights: null router, norm or shared-gate pointer");
+  if (reinterpret_cast<uintptr_t>(w->router) % 16 != 0)
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "router: device pointer must be 16-byte aligned");
+  return XABE_OK;
+}
+
 static int shared_fp32(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
                        xabe_quant_tensor up, xabe_quant_tensor down, const float* x, float* out) {
   const xabe_moe_geometry& g = k->g;

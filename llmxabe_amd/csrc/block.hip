@@ -78,6 +78,7 @@ int xabe_moe_block_forward_stage(xabe_moe_block* blk, void* stream, const xabe_m
   XABE_TRY(blk_check_len("l_out", blk->n_act, l_out_len));
   if (!decode_block_supported(blk->moe, blk->buffers, w))
     return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "forward_stage: this geometry does not take the three-launch decode path");
+  XABE_TRY(check_layer_stacks(blk->moe, w));
   return launch_decode_block(blk->moe, as_stream(stream), blk->buffers, w, residual, logit_bias, blk->eps, blk->normed,
                              blk->logits, blk->shexp, blk->gate, blk->routed, ffn_out, l_out, 1u << stage);
 }
@@ -95,9 +96,11 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
   XABE_TRY(xabe_moe_block_publish_tokens(blk, stream, tokens));
 
   // decode widths, model shapes: the eight steps below regrouped into three launches, same arithmetic
-  if (blk->fused_decode && !blk->moe->exact_regime && decode_block_supported(blk->moe, blk->buffers, w))
+  if (blk->fused_decode && !blk->moe->exact_regime && decode_block_supported(blk->moe, blk->buffers, w)) {
+    XABE_TRY(check_layer_stacks(blk->moe, w));  // (the checks the step-by-step sequence below makes call by call)
     return launch_decode_block(blk->moe, as_stream(stream), blk->buffers, w, residual, logit_bias, blk->eps, blk->normed,
                                blk->logits, blk->shexp, blk->gate, blk->routed, ffn_out, l_out);
+  }
 
   // 1. post-mixer RMSNorm over every row of the buffer
   XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,

@@ -56,6 +56,9 @@ int pick_tile_rows(const xabe_moe_kernels* k, size_t live_units, int n_rows, int
 
 // the decode-width block in three launches (decode_block.hip)
 bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, const xabe_moe_layer_weights* w);
+// the checks the step-by-step entry points make on a layer's six stacks (whole blocks, element counts, formats,
+// 16-byte-aligned device pointers), for the block-level paths that launch without passing through them (api.hip)
+int check_layer_stacks(const xabe_moe_kernels* k, const xabe_moe_layer_weights* w);
 int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, const xabe_moe_layer_weights* w,
                         const float* residual, const float* logit_bias, float eps, float* normed, float* logits,
                         float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches = 7u);
