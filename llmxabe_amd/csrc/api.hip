@@ -148,6 +148,19 @@ static bool launch_block_resident(Shape shape, const ExpertArgs& a, size_t units
   return true;
 }
 
+template <int Q, int NM, int R, int TOK, bool RESID>
+static bool launch_long_rows_lds(const LongRowArgs& la, dim3 grid, dim3 block, size_t smem, hipStream_t s) {
+  auto kern = k_shared_long_rows<Q, NM, R, TOK, RESID, true>;
+  static size_t allowed = 0;  // per instantiation; the attribute is per function, raised when a launch needs more
+  if (smem > allowed) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return false;
+    allowed = smem;
+  }
+  hipLaunchKernelGGL(kern, grid, block, smem, s, la);
+  return true;
+}
+
 // Rows longer than one step, no expert indirection (dense sibling, wide shared experts): the step-outer
 // kernel, R rows per wavefront (2 for a gate/up pair, 4 for one matrix).  `la.l_out` set: add the residual
 // in the epilogue.
@@ -170,6 +183,21 @@ bool launch_long_rows(const xabe_moe_kernels* k, int quant, int nm, const LongRo
   const size_t row_bytes = (size_t)a.K / xabe_expert_quant_block_elements(quant) * xabe_expert_quant_block_bytes(quant);
   auto on16 = [&](const uint8_t* w) { return !w || (reinterpret_cast<uintptr_t>(w) % 16 == 0 && ((size_t)a.n_rows * row_bytes) % 16 == 0); };
   if (!(on16(a.w0) && on16(a.w1))) return false;
+  // Three tokens or more, gate/up: four tokens per pass with the activation rows in LDS (the kernel's XLDS form),
+  // where four rows and eight wavefronts' staging slots fit; eight wavefronts per workgroup, one workgroup per
+  // CU and pass, persistent over the row groups.  (Down's rows are too long for four of them to fit.)
+  if (nm == 2 && k->g.max_tokens >= 3 && a.K % 4 == 0) {
+    const int tokx = 4;
+    const unsigned wv = 8;
+    const size_t slot = (size_t)r * nm * (quant == XABE_QUANT_Q6K ? StageFmt<kQ6K>::kSlotBytes : StageFmt<kQ8_0>::kSlotBytes);
+    const size_t smem = (size_t)tokx * a.K * sizeof(float) + wv * slot;
+    if (smem <= 159 * 1024) {
+      const unsigned passx = (unsigned)((k->g.max_tokens + tokx - 1) / tokx);
+      dim3 gridx((unsigned)std::min<size_t>(((size_t)groups + wv - 1) / wv, (size_t)k->num_cus), passx), blockx(64 * wv);
+      if (quant == XABE_QUANT_Q6K) return launch_long_rows_lds<kQ6K, 2, 2, 4, false>(la, gridx, blockx, smem, s);
+      return launch_long_rows_lds<kQ8_0, 2, 2, 4, false>(la, gridx, blockx, smem, s);
+    }
+  }
 #define XABE_LONG4(Q, TOK, R)                                                                                    \
   do {                                                                                                            \
     if (nm == 2) hipLaunchKernelGGL((k_shared_long_rows<Q, 2, R, TOK, false>), grid, block, 0, s, la);            \

@@ -618,12 +618,18 @@ struct LongRowArgs {
   float* l_out;           // RESID
 };
 
-template <int QUANT, int NM, int R, int TOK, bool RESID>
-__global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
+//   XLDS:   the pass's activation rows are copied into LDS once per workgroup and every step reads its 32
+//           elements per token and lane from there, just before they are used: no activation registers held
+//           across a step, which is what lets a pass serve four tokens (each weight dequantised once for the
+//           four) where the register form stops at two.  Workgroups of up to eight wavefronts, persistent over
+//           the row groups; dynamic LDS = TOK * K floats, then the wavefronts' staging slots.
+template <int QUANT, int NM, int R, int TOK, bool RESID, bool XLDS = false>
+__global__ void __launch_bounds__(XLDS ? 512 : 256) k_shared_long_rows(LongRowArgs la) {
   using F = Fmt<QUANT>;
   using Raw = typename F::Raw;
   constexpr int kSlot = StageFmt<QUANT>::kSlotBytes;
-  __shared__ __attribute__((aligned(16))) uint8_t s_slots[kWavesPerWg * R * NM * kSlot];
+  __shared__ __attribute__((aligned(16))) uint8_t s_slots_static[XLDS ? 16 : kWavesPerWg * R * NM * kSlot];
+  extern __shared__ __attribute__((aligned(16))) float s_xrows[];
   const ExpertArgs& a = la.m;
   const int valid = *a.valid_tokens;
   const int t0 = blockIdx.y * TOK;
@@ -633,7 +639,19 @@ __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const size_t row_bytes = (size_t)(a.K / F::kBlockElems) * F::kBlockBytes;
   const int steps = (a.K + kStepElems - 1) / kStepElems;
-  const int wg_waves = (int)(blockDim.x >> 6);  // 4, or 1 for a matrix with few row groups
+  const int wg_waves = (int)(blockDim.x >> 6);  // 4, or 1 for a matrix with few row groups (XLDS: up to 8)
+  uint8_t* const s_slots = XLDS ? reinterpret_cast<uint8_t*>(s_xrows + (size_t)TOK * a.K) : s_slots_static;
+  if constexpr (XLDS) {
+    // (a token past the batch copies the last live one: computed, never stored)
+    const int n4 = a.K / 4;
+#pragma unroll
+    for (int t = 0; t < TOK; ++t) {
+      const float4* src = reinterpret_cast<const float4*>(a.x + (size_t)(t0 + min(t, nt - 1)) * a.K);
+      float4* dst = reinterpret_cast<float4*>(s_xrows + (size_t)t * a.K);
+      for (int i = threadIdx.x; i < n4; i += blockDim.x) dst[i] = src[i];
+    }
+    __syncthreads();
+  }
 #pragma unroll 1
   for (int rg = (int)blockIdx.x * wg_waves + wave; rg < a.n_rows / R; rg += (int)gridDim.x * wg_waves) {
     const int row0 = rg * R;
@@ -644,12 +662,13 @@ __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
       for (int m = 0; m < NM; ++m)
 #pragma unroll
         for (int t = 0; t < TOK; ++t) acc[r][m][t] = 0.0f;
-    float x[TOK][32];
+    float x[XLDS ? 1 : TOK][32];
     Staged<QUANT> pend[R][NM];
     // raw activations of step k.  Unconditional loads from clamped addresses (a token past the batch reads
     // the last live one, a lane past the end of the row its last block): a select here would need the data
     // at once and stall the pipeline; lanes past the row are zeroed where the values are used.
     auto issue_x = [&](int k) __attribute__((always_inline)) {
+      if constexpr (XLDS) return;
       const int koff = min(lane_koff<QUANT, 1>(g, k), a.K - F::kBlockElems);
 #pragma unroll
       for (int t = 0; t < TOK; ++t) lane_x_load<QUANT>(a.x + (size_t)(t0 + min(t, nt - 1)) * a.K, koff, g, x[t]);
@@ -672,11 +691,13 @@ __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
     for (int k = 0; k < steps; ++k) {
       const bool act = lane_koff<QUANT, 1>(g, k) < a.K;
       float xl[TOK][32], xs[TOK][4];
+      if constexpr (!XLDS) {
 #pragma unroll
-      for (int t = 0; t < TOK; ++t) {
+        for (int t = 0; t < TOK; ++t) {
 #pragma unroll
-        for (int i = 0; i < 32; ++i) xl[t][i] = act ? x[t][i] : 0.0f;
-        lane_x_offsets<QUANT>(xl[t], xs[t]);
+          for (int i = 0; i < 32; ++i) xl[t][i] = act ? x[t][i] : 0.0f;
+          lane_x_offsets<QUANT>(xl[t], xs[t]);
+        }
       }
       Raw raw[R][NM];
 #pragma unroll
@@ -685,6 +706,17 @@ __global__ void __launch_bounds__(256) k_shared_long_rows(LongRowArgs la) {
         for (int m = 0; m < NM; ++m)
           stage_pick<QUANT>(pend[r][m], s_slots + (size_t)((wave * R + r) * NM + m) * kSlot, act, g, raw[r][m]);
       if (k + 1 < steps) issue_w(k + 1);
+      if constexpr (XLDS) {
+        // the step's activations, out of LDS, once the staging registers above have been handed back
+        const int koff = min(lane_koff<QUANT, 1>(g, k), a.K - F::kBlockElems);
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) {
+          lane_x_load<QUANT>(s_xrows + (size_t)t * a.K, koff, g, xl[t]);
+#pragma unroll
+          for (int i = 0; i < 32; ++i) xl[t][i] = act ? xl[t][i] : 0.0f;
+          lane_x_offsets<QUANT>(xl[t], xs[t]);
+        }
+      }
 #pragma unroll
       for (int r = 0; r < R; ++r)
 #pragma unroll
