@@ -244,7 +244,8 @@ def main() -> int:
 
 MFMA_PEAK_TFLOPS = 2500.0
 # name -> (kind, tokens, layers rotated): the MoE block at other widths and the dense sibling
-OTHER_WORKLOADS = {"decode_b32": ("moe", 32, 16), "prefill_512": ("moe", 512, 4), "prefill_8192": ("moe", 8192, 2),
+OTHER_WORKLOADS = {"decode_b32": ("moe", 32, 16), "prefill_512": ("moe", 512, 4), "prefill_512_uniform": ("moe", 512, 4),
+                   "prefill_8192": ("moe", 8192, 2),
                    "dense_b1": ("dense", 1, 4), "dense_b8": ("dense", 8, 4), "dense_2048": ("dense", 2048, 2),
                    # the LM head (2048 -> 248 320, Q8_0: 540 MB per pass), two copies rotated
                    "lm_head_b1": ("lm_head", 1, 2), "lm_head_b3": ("lm_head", 3, 2), "lm_head_b8": ("lm_head", 8, 2)}
@@ -280,6 +281,12 @@ def other_workload(args) -> int:
         width = H
     x = X.synth_normal_f32(99, T * width, 1.0).view(T, width)
     ffn_out, l_out = torch.zeros_like(x), torch.zeros_like(x)
+    extra = {}
+    if args.workload == "prefill_512":
+        # the skewed configuration: a seeded Zipf(s = 1.1) bias over the experts, added to the router logits before
+        # routing (b_e = -s ln(rank_e) over a seeded permutation of the experts, i.e. selection odds proportional to rank^-1.1)
+        rank = np.random.default_rng(5).permutation(256) + 1
+        extra["logit_bias"] = torch.from_numpy((-1.1 * np.log(rank)).astype(np.float32)).cuda()
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()
     reps_w = max(1, min(args.warmup, 64) // L)
@@ -287,13 +294,13 @@ def other_workload(args) -> int:
     with torch.cuda.stream(stream):
         for _ in range(reps_w):
             for i in range(L):
-                blk.forward(layers[i], x, T, ffn_out, l_out)
+                blk.forward(layers[i], x, T, ffn_out, l_out, **extra)
         stream.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
         for _ in range(reps):
             for i in range(L):
-                blk.forward(layers[i], x, T, ffn_out, l_out)
+                blk.forward(layers[i], x, T, ffn_out, l_out, **extra)
         e1.record(stream)
         e1.synchronize()
     steps = reps * L
@@ -305,7 +312,11 @@ def other_workload(args) -> int:
         flops = T * 57671680
         cfg = {"workload": "moe_block_" + args.workload, "tokens": T, "num_experts": 256, "top_k": 8, "hidden": 2048,
                "intermediate": 512, "expert_quant": "Q6_K", "shared_and_router_quant": "Q8_0", "layers_rotated": L,
-               "launch": "eager", "distinct_experts": distinct}
+               "launch": "eager", "distinct_experts": distinct,
+               "router_bias": "zipf s=1.1 (b_e = -1.1 ln rank_e), seed 5" if extra else None}
+        if extra:
+            counts = np.bincount(ids.ravel(), minlength=256)
+            cfg["expert_load"] = {"max": int(counts.max()), "experts_with_at_most_2_tokens": int((counts <= 2).sum())}
     else:
         byts = 3 * 5120 * 17408 // 256 * 210
         flops = T * 3 * 2 * 5120 * 17408
