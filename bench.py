@@ -246,6 +246,8 @@ MFMA_PEAK_TFLOPS = 2500.0
 # name -> (kind, tokens, layers rotated): the MoE block at other widths and the dense sibling
 OTHER_WORKLOADS = {"decode_b32": ("moe", 32, 16), "prefill_512": ("moe", 512, 4), "prefill_512_uniform": ("moe", 512, 4),
                    "prefill_8192": ("moe", 8192, 2),
+                   # the 40-layer stack (26.4 GB of experts resident), each block's l_out the next block's input
+                   "stack40_b32": ("stack", 32, 40), "stack40_8192": ("stack", 8192, 40),
                    "dense_b1": ("dense", 1, 4), "dense_b8": ("dense", 8, 4), "dense_2048": ("dense", 2048, 2),
                    # the LM head (2048 -> 248 320, Q8_0: 540 MB per pass), two copies rotated
                    "lm_head_b1": ("lm_head", 1, 2), "lm_head_b3": ("lm_head", 3, 2), "lm_head_b8": ("lm_head", 8, 2)}
@@ -264,6 +266,8 @@ def other_workload(args) -> int:
     kind, T, L = OTHER_WORKLOADS[args.workload]
     if kind == "lm_head":
         return lm_head_workload(args, T, L)
+    if kind == "stack":
+        return stack_workload(args, T, L)
     if kind == "moe":
         g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
         layers = [make_layer_device_only(X, g, seed=10_000 + 100 * l) for l in range(L)]
@@ -334,6 +338,74 @@ def other_workload(args) -> int:
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if T >= 64 else "f32",
         "data": "synthetic", "config": cfg, "roofline": roof, "algorithmic_bytes_per_step": byts, "flops_per_step": flops,
         "cpu_baseline": None}))
+    return 0
+
+
+def stack_workload(args, T, L) -> int:
+    """L independently seeded MoE layers resident at once, one pass of T tokens through all of them per step:
+    layer l's l_out (residual + block output; the RMSNorm is the next block's first step) is layer l + 1's
+    input.  Ping-pong activation buffers, eager launches, HIP events on the launch stream."""
+    import numpy as np
+    import torch
+
+    import llmxabe_amd as X
+
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
+    layers = [make_layer_device_only(X, g, seed=20_000 + 100 * l) for l in range(L)]
+    blk = X.MoeBlock(g)
+    blk.publish_tokens(T)
+    x0 = X.synth_normal_f32(99, T * 2048, 1.0).view(T, 2048)
+    bufs = [torch.zeros_like(x0), torch.zeros_like(x0)]
+    ffn_out = torch.zeros_like(x0)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+
+    def one_pass():
+        cur = x0
+        for i, w in enumerate(layers):
+            nxt = bufs[i & 1]
+            blk.forward(w, cur, T, ffn_out, nxt)
+            cur = nxt
+        return cur
+
+    reps_w, reps = max(1, min(args.warmup, 4)), max(1, min(args.steps, 16 if T < 512 else 4))
+    with torch.cuda.stream(stream):
+        for _ in range(reps_w):
+            one_pass()
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            out = one_pass()
+        e1.record(stream)
+        e1.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    finite = bool(torch.isfinite(out).all().item())
+    flops = L * T * 57671680
+    weight_bytes = L * (256 * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES)
+    tflops = flops / (ms * 1e-3) / 1e12
+    mfma = T >= 64
+    # algorithmic bytes of a pass: every layer's distinct selected experts (read back layer by layer, untimed)
+    byts, cur = 0, x0
+    for i, w in enumerate(layers):
+        blk.forward(w, cur, T, ffn_out, bufs[i & 1])
+        cur = bufs[i & 1]
+        distinct = len(np.unique(blk.buffers().topk_ids().cpu().numpy().reshape(T, 8)))
+        byts += distinct * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES + 16384 + T * 2048 * 4 * 3
+    gbps = byts / (ms * 1e-3) / 1e9
+    roof = ({"kernel": "whole stack", "bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+             "frac": tflops / MFMA_PEAK_TFLOPS, "traffic": None} if mfma else
+            {"kernel": "whole stack", "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": gbps / HBM_PEAK_GBPS, "traffic": None})
+    print(json.dumps({
+        "metric": "MoE-block tokens/s at 1 GPU; decode HBM GB/s %peak; prefill MFMA util %", "value": T / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": reps, "warmup": reps_w, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if mfma else "f32", "data": "synthetic",
+        "config": {"workload": "moe_stack_" + args.workload, "layers": L, "tokens": T, "num_experts": 256, "top_k": 8,
+                   "hidden": 2048, "intermediate": 512, "expert_quant": "Q6_K", "shared_and_router_quant": "Q8_0",
+                   "resident_weight_bytes": weight_bytes, "launch": "eager", "us_per_layer": ms * 1e3 / L,
+                   "output_finite": finite},
+        "roofline": roof, "algorithmic_bytes_per_step": byts, "flops_per_step": flops, "cpu_baseline": None}))
     return 0
 
 
