@@ -35,7 +35,13 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kBM = 128;          // token rows per tile (64 in the narrow form: see k_mfma_expert's TBM)
 constexpr int kBR = 128;          // weight rows per tile
 constexpr int kBK = 128;          // contraction elements per step
-constexpr int kLd = kBK + 8;      // LDS row stride of the weight tile in halfs (272 B: 16-B reads are conflict-free)
+// The weight tile's rows are unpadded too, its 16-byte chunks XOR-swizzled by w_swizzle(row): any eight
+// consecutive rows spread one chunk over the eight 16-byte slots of a 128-byte bank line (the fragment reads:
+// lanes = rows), and two neighbouring rows put chunks 4j .. 4j + 3 into disjoint halves of it (the
+// dequantised stores: eight lanes = two rows x four units).  With padded rows (272 B) the reads were
+// conflict-free and the stores two-way conflicted: a fifth of the LDS cycles the counters showed; the bank
+// conflict counter now reads zero (the launches take the same time: LDS was not what held them).
+constexpr int kLd = kBK;
 // The activation tile goes from global memory straight into LDS (global_load_lds_dwordx4: no registers, no
 // store instructions), which writes a wavefront's 64 pieces contiguously, so its rows are unpadded (256 B)
 // and the 16-byte chunks of a row are stored XOR-swizzled by the row number instead: chunk c of row r sits at
@@ -59,6 +65,10 @@ struct MfmaArgs {
   int top_k;
 };
 
+__device__ __forceinline__ int w_swizzle(int row) {
+  return (row & 8) | ((row & 1) << 2) | ((row >> 1) & 3);
+}
+
 // ---- prologues: one 32-element unit of one weight row -> 32 halfs in LDS -----------------
 __device__ __forceinline__ u32x4 pack8(uint32_t c0, uint32_t c1, half2v off, half2v s) {
   // c0, c1: eight byte codes; returns eight halfs (code + 1024 - off) * s
@@ -79,7 +89,7 @@ __device__ __forceinline__ u32x4 pack8(uint32_t c0, uint32_t c1, half2v off, hal
 }
 
 // Q6_K unit (half h of a superblock, l8): codes at j*32 + l8*8 + i of that half.
-__device__ __forceinline__ void q6_unit_to_lds(const Q6Raw& r, int l8, _Float16* brow) {
+__device__ __forceinline__ void q6_unit_to_lds(const Q6Raw& r, int l8, _Float16* brow, int swz) {
   const int is8 = (l8 >> 1) * 8;
   const uint32_t slo = r.sc0 >> is8, shi = r.sc1 >> is8;
   const float d = f16_bits_to_f32(r.dh) * kWScale;
@@ -99,18 +109,18 @@ __device__ __forceinline__ void q6_unit_to_lds(const Q6Raw& r, int l8, _Float16*
   for (int j = 0; j < 4; ++j) {
     const _Float16 sh = (_Float16)ds[j];
     const half2v s = {sh, sh};
-    *reinterpret_cast<u32x4*>(brow + j * 32 + l8 * 8) = pack8(c[0][j], c[1][j], off, s);
+    *reinterpret_cast<u32x4*>(brow + ((j * 4 + l8) ^ swz) * 8) = pack8(c[0][j], c[1][j], off, s);
   }
 }
 
-// Q8_0 unit: one 34-byte block -> 32 consecutive halfs.
-__device__ __forceinline__ void q8_unit_to_lds(const Q8Raw& r, _Float16* bdst) {
+// Q8_0 unit: one 34-byte block -> the row's chunks 4 du .. 4 du + 3.
+__device__ __forceinline__ void q8_unit_to_lds(const Q8Raw& r, int du, _Float16* brow, int swz) {
   const _Float16 sh = (_Float16)(f16_bits_to_f32(r.dh) * kWScale);  // exact: d is fp16, scaled by 2^8
   const half2v s = {sh, sh};
   const half2v off = {(_Float16)-1152.0f, (_Float16)-1152.0f};      // 1024 (perm bias) + 128 (sign flip)
 #pragma unroll
   for (int w = 0; w < 4; ++w)
-    reinterpret_cast<u32x4*>(bdst)[w] = pack8(r.q[2 * w] ^ 0x80808080u, r.q[2 * w + 1] ^ 0x80808080u, off, s);
+    *reinterpret_cast<u32x4*>(brow + ((du * 4 + w) ^ swz) * 8) = pack8(r.q[2 * w] ^ 0x80808080u, r.q[2 * w + 1] ^ 0x80808080u, off, s);
 }
 
 // Nothing moves across this point, in either direction, when the compiler schedules.
@@ -209,7 +219,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   static_assert(TBM == 128 || TBM == 64, "token tile");
   constexpr int MI = TBM / 64;       // 32-row blocks of the tile per wavefront
   constexpr int kAPieces = TBM / 16; // 16-byte activation pieces per thread and step
-  // 70.5 KB of LDS per workgroup (two per CU): dynamic, since the static limit is 64 KB
+  // 67.5 KB of LDS per workgroup at 128 token rows (two per CU): dynamic, since the static limit is 64 KB
   extern __shared__ __attribute__((aligned(16))) uint8_t mfma_smem[];
   _Float16* sA = reinterpret_cast<_Float16*>(mfma_smem);
   _Float16* sB = sA + TBM * kLdA;
@@ -423,11 +433,11 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
         if constexpr (QUANT == kQ6K) {
           Q6Raw r;
           q6_finish(w[P].u[i], r);
-          q6_unit_to_lds(r, du, &sB[rb * kLd]);
+          q6_unit_to_lds(r, du, &sB[rb * kLd], w_swizzle(rb));
         } else {
           Q8Raw r;
           q8_finish(w[P].u[i], r);
-          q8_unit_to_lds(r, &sB[rb * kLd + du * 32]);
+          q8_unit_to_lds(r, du, &sB[rb * kLd], w_swizzle(rb));
         }
       }
       if (ks == nks - 1 && has_next && tid < TBM) {
@@ -459,7 +469,8 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       if (ks + 1 == nks && has_next) set_arow(buf ^ 1);
       const _Float16* pa = &sA[(wm * (TBM / 2) + (lane & 31)) * kLdA];
       const int swz = lane & 15, khalf = lane >> 5;  // (the row's low four bits are the lane's)
-      const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd + (lane >> 5) * 8];
+      const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd];
+      const int wswz = w_swizzle(lane & 15);  // (the rows' low four bits are the lane's)
       // Operand fragments one sub-step ahead, in two register sets: the four LDS reads of sub-step kk + 1 are
       // issued before the four matrix instructions of sub-step kk, so their latency hides behind 128 cycles of
       // matrix work instead of standing between every group of four.
@@ -468,8 +479,9 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
         const int apos = ((kk * 2 + khalf) ^ swz) * 8;
         fa[set][0] = *reinterpret_cast<const half8*>(pa + apos);
         if constexpr (MI == 2) fa[set][MI - 1] = *reinterpret_cast<const half8*>(pa + 32 * kLdA + apos);
-        fb[set][0] = *reinterpret_cast<const half8*>(pb + kk * 16);
-        fb[set][1] = *reinterpret_cast<const half8*>(pb + 32 * kLd + kk * 16);
+        const int bpos = ((kk * 2 + khalf) ^ wswz) * 8;
+        fb[set][0] = *reinterpret_cast<const half8*>(pb + bpos);
+        fb[set][1] = *reinterpret_cast<const half8*>(pb + 32 * kLd + bpos);
       };
       frags(0, 0);
 #pragma unroll
@@ -640,7 +652,7 @@ static int shared_tile_rows(const xabe_moe_kernels* k, size_t row_tiles) {
 
 template <int NM, bool ROUTED, int TBM>
 static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
-  // workgroups resident per CU: the narrow tile's registers (about 150) and LDS (51.5 KB) leave room for a third
+  // workgroups resident per CU: the narrow tile's registers (about 150) and LDS (49.5 KB) leave room for a third
   const size_t per_cu = TBM == 64 ? 3 : 2;
   const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * per_cu));
   constexpr size_t smem = (size_t)(TBM * kLdA + kBR * kLd) * sizeof(_Float16) + 2 * 3 * TBM * sizeof(int);
