@@ -148,17 +148,21 @@ static bool launch_block_resident(Shape shape, const ExpertArgs& a, size_t units
   return true;
 }
 
+constexpr size_t kLongRowsLdsMax = 159 * 1024;  // what a workgroup of the LDS-activation form may ask for
 template <int Q, int NM, int R, int TOK, bool RESID>
 static bool launch_long_rows_lds(const LongRowArgs& la, dim3 grid, dim3 block, size_t smem, hipStream_t s) {
-  auto kern = k_shared_long_rows<Q, NM, R, TOK, RESID, true>;
-  static size_t allowed = 0;  // per instantiation; the attribute is per function, raised when a launch needs more
-  if (smem > allowed) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-      return false;
-    allowed = smem;
-  }
-  hipLaunchKernelGGL(kern, grid, block, smem, s, la);
+  hipLaunchKernelGGL((k_shared_long_rows<Q, NM, R, TOK, RESID, true>), grid, block, smem, s, la);
   return true;
+}
+int long_rows_configure() {
+  static bool done = false;  // (one device per process)
+  if (done) return XABE_OK;
+  const void* fns[2] = {reinterpret_cast<const void*>(k_shared_long_rows<kQ6K, 2, 2, 4, false, true>),
+                        reinterpret_cast<const void*>(k_shared_long_rows<kQ8_0, 2, 2, 4, false, true>)};
+  for (const void* f : fns)
+    XABE_HIP_TRY(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongRowsLdsMax));
+  done = true;
+  return XABE_OK;
 }
 
 // Rows longer than one step, no expert indirection (dense sibling, wide shared experts): the step-outer
@@ -191,7 +195,7 @@ bool launch_long_rows(const xabe_moe_kernels* k, int quant, int nm, const LongRo
     const unsigned wv = 8;
     const size_t slot = (size_t)r * nm * (quant == XABE_QUANT_Q6K ? StageFmt<kQ6K>::kSlotBytes : StageFmt<kQ8_0>::kSlotBytes);
     const size_t smem = (size_t)tokx * a.K * sizeof(float) + wv * slot;
-    if (smem <= 159 * 1024) {
+    if (smem <= kLongRowsLdsMax) {
       const unsigned passx = (unsigned)((k->g.max_tokens + tokx - 1) / tokx);
       dim3 gridx((unsigned)std::min<size_t>(((size_t)groups + wv - 1) / wv, (size_t)k->num_cus), passx), blockx(64 * wv);
       if (quant == XABE_QUANT_Q6K) return launch_long_rows_lds<kQ6K, 2, 2, 4, false>(la, gridx, blockx, smem, s);
@@ -416,6 +420,13 @@ int xabe_moe_kernels_new(const xabe_moe_geometry* geometry, xabe_moe_kernels** o
   k->force_community = false;
   k->device = dev;
   k->num_cus = prop.multiProcessorCount;
+  // everything one-time happens here, none of it on the launch path (launches are captured into graphs)
+  int st = mfma_configure();
+  if (st == XABE_OK) st = long_rows_configure();
+  if (st != XABE_OK) {
+    delete k;
+    return st;
+  }
   *out = k;
   return XABE_OK;
 }

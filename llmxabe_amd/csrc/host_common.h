@@ -73,6 +73,9 @@ int dense_fp32_fused(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers*
 bool router_gemm_supported(const xabe_moe_kernels* k, int router_quant);
 int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,
                        int router_quant, const float* normed, float* logits);
+// one-time, at handle creation: LDS limits of the kernels that ask for more than the static 64 KB (mfma.hip, api.hip)
+int mfma_configure();
+int long_rows_configure();
 bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int gate_q, int up_q, int down_q, bool routed);
 int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
                                  xabe_quant_tensor up, xabe_quant_tensor down, const float* x);

@@ -650,22 +650,43 @@ static int shared_tile_rows(const xabe_moe_kernels* k, size_t row_tiles) {
   return (k->g.max_tokens + 63) / 64 * row_tiles <= (size_t)k->num_cus * 2 ? 64 : kBM;
 }
 
+// LDS a workgroup of the kernel asks for (dynamic: above the static limit).  The limit is raised per function,
+// once, when a kernels handle is created (mfma_configure): nothing on the launch path but the launch.
+template <int TBM>
+constexpr size_t mfma_lds_bytes() {
+  return (size_t)(TBM * kLdA + kBR * kLd) * sizeof(_Float16) + 2 * 3 * TBM * sizeof(int);
+}
+template <int NM, bool ROUTED, int TBM>
+static int configure_one() {
+  const void* fns[2] = {reinterpret_cast<const void*>(k_mfma_expert<kQ6K, NM, ROUTED, TBM>),
+                        reinterpret_cast<const void*>(k_mfma_expert<kQ8_0, NM, ROUTED, TBM>)};
+  for (const void* f : fns)
+    XABE_HIP_TRY(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)mfma_lds_bytes<TBM>()));
+  return XABE_OK;
+}
+int mfma_configure() {
+  static bool done = false;  // (one device per process)
+  if (done) return XABE_OK;
+  XABE_TRY((configure_one<1, false, 64>()));
+  XABE_TRY((configure_one<1, false, 128>()));
+  XABE_TRY((configure_one<1, true, 64>()));
+  XABE_TRY((configure_one<1, true, 128>()));
+  XABE_TRY((configure_one<2, false, 64>()));
+  XABE_TRY((configure_one<2, false, 128>()));
+  XABE_TRY((configure_one<2, true, 64>()));
+  XABE_TRY((configure_one<2, true, 128>()));
+  done = true;
+  return XABE_OK;
+}
+
 template <int NM, bool ROUTED, int TBM>
 static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
   // workgroups resident per CU: the narrow tile's registers (about 150) and LDS (49.5 KB) leave room for a third
   const size_t per_cu = TBM == 64 ? 3 : 2;
   const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * per_cu));
-  constexpr size_t smem = (size_t)(TBM * kLdA + kBR * kLd) * sizeof(_Float16) + 2 * 3 * TBM * sizeof(int);
-  auto kq6 = k_mfma_expert<kQ6K, NM, ROUTED, TBM>;
-  auto kq8 = k_mfma_expert<kQ8_0, NM, ROUTED, TBM>;
-  static bool configured = false;  // per instantiation; the attribute is per function, set once
-  if (!configured) {
-    XABE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kq6), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    XABE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kq8), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    configured = true;
-  }
-  if (quant == XABE_QUANT_Q6K) hipLaunchKernelGGL(kq6, dim3(grid), dim3(256), smem, s, a);
-  else hipLaunchKernelGGL(kq8, dim3(grid), dim3(256), smem, s, a);
+  constexpr size_t smem = mfma_lds_bytes<TBM>();
+  if (quant == XABE_QUANT_Q6K) hipLaunchKernelGGL((k_mfma_expert<kQ6K, NM, ROUTED, TBM>), dim3(grid), dim3(256), smem, s, a);
+  else hipLaunchKernelGGL((k_mfma_expert<kQ8_0, NM, ROUTED, TBM>), dim3(grid), dim3(256), smem, s, a);
   XABE_HIP_TRY(hipGetLastError());
   return XABE_OK;
 }

@@ -72,6 +72,17 @@ def test_dense_block_and_lm_head_replay(oracle, X):
     _replays(torch, stream, lambda: blk.forward(w, x, 2, ffn, lout), [ffn, lout],
              lambda: (ffn.zero_(), lout.zero_()), want, "dense block")
 
+    # eight tokens: gate/up takes four tokens per pass with the activation rows in LDS (a launch that asks for
+    # more than the static LDS limit; the limit is raised when the block is created, not on the launch path)
+    blk8 = X.DenseFfnBlock(H, I, 8)
+    x8 = X.synth_normal_f32(52, 8 * H, 1.0).view(8, H)
+    ffn8, lout8 = torch.zeros_like(x8), torch.zeros_like(x8)
+    blk8.forward(w, x8, 7, ffn8, lout8)
+    torch.cuda.synchronize()
+    want8 = [ffn8.view(torch.int32).clone(), lout8.view(torch.int32).clone()]
+    _replays(torch, stream, lambda: blk8.forward(w, x8, 7, ffn8, lout8), [ffn8, lout8],
+             lambda: (ffn8.fill_(float("nan")), lout8.fill_(float("nan"))), want8, "dense block, 7 of 8 tokens", rows=7)
+
     g = X.LmHeadGeometry(2048, 8192, 3)
     k = X.LmHeadKernels(g)
     head = X.HeadTensor.q8_0(X.synth_quant(X.ExpertQuant.Q8_0, 61, g.elements(), 0.02))
