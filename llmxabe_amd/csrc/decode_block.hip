@@ -40,6 +40,11 @@ namespace xabe {
 constexpr size_t kDecodeBlockMaxTokens = 16;  // widest batch served by the three launches (the dispatch-table regime is faster from ~24 tokens)
 constexpr int kMaxTopK = 8;       // contributions held in registers by k_decode_down
 constexpr int kMaxInter = 512;    // intermediate width staged in LDS by k_decode_down
+// Steps per wavefront of the first launch: a wavefront reads 24 KB of activation rows and norm weights for the 2-4 KB
+// of weights of one step, so more steps against the same registers cut what the launch pulls out of L2, at the
+// price of fewer workgroups.  Measured per width (launch A, us, depth 1 / 2 / 4): one token 5.2 / 5.3 / 6.6, three
+// 7.7 / 6.5 / 8.4, eight 14.2 / 9.4 / 8.4, sixteen - / 15.7 / 11.7.
+static int logits_depth(int max_tokens) { return max_tokens <= 1 ? 1 : max_tokens <= 6 ? 2 : 4; }
 
 #ifdef XABE_TRACE_ITEMS
 // measurement builds only: per-workgroup timestamps (100 MHz device clock), [kernel][workgroup][slot]
@@ -82,7 +87,7 @@ struct DecodeArgs {
 // One step (RPS rows of K = 2048 / RPS elements) of a matrix, or of a gate/up pair, against TC tokens whose
 // rows are normalised on load.  Issues every load before the first use.
 //   NM = 2: out[t][row] = silu(gate . x_t) * (up . x_t);   NM = 1: out[t][row] = (w . x_t) (+ bias[row]).
-template <int QUANT, int RPS, int TC, int NM>
+template <int QUANT, int RPS, int TC, int NM, int D = 1>
 __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, int K,
                                             int n_rows, int row0, const float* const (&xrow)[TC],
                                             const float* __restrict__ norm_w, float eps, float* const (&out)[TC],
@@ -107,9 +112,14 @@ __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, cons
 #pragma unroll
   for (int t = 0; t < TC; ++t) lane_x_load<QUANT>(xrow[t], koff, g, x[t]);
   lane_x_load<QUANT>(norm_w, koff, g, nw);
-  Raw r[NM];
-  load_raw<QUANT, true>(w0 + (size_t)row0 * row_bytes, true, g, r[0]);
-  if constexpr (NM == 2) load_raw<QUANT, true>(w1 + (size_t)row0 * row_bytes, true, g, r[NM - 1]);
+  // D steps (RPS rows each) against the same activation registers: the rows' weights are all requested here
+  Raw r[D][NM];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    const int rd = min(row0 + d * RPS, n_rows - RPS);  // (a step past the matrix re-reads its last one: never stored)
+    load_raw<QUANT, true>(w0 + (size_t)rd * row_bytes, true, g, r[d][0]);
+    if constexpr (NM == 2) load_raw<QUANT, true>(w1 + (size_t)rd * row_bytes, true, g, r[d][NM - 1]);
+  }
 #pragma unroll
   for (int t = 0; t < TC; ++t) {
     float s = 0.0f;
@@ -125,25 +135,28 @@ __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, cons
     for (int i = 0; i < 32; ++i) x[t][i] = x[t][i] * inv * nw[i];
     lane_x_offsets<QUANT>(x[t], xs[t]);
   }
-  float tot[NM][TC];
-#pragma unroll
-  for (int m = 0; m < NM; ++m) {
-#pragma unroll
-    for (int t = 0; t < TC; ++t) tot[m][t] = 0.0f;
-    accum<QUANT, TC>(r[m], g, x, xs, tot[m]);
-#pragma unroll
-    for (int t = 0; t < TC; ++t) tot[m][t] = group_sum<G>(tot[m][t]);
-  }
   // the live-token count was requested first and is only needed here: rows past it were computed from
   // whatever the buffer held (in bounds, sized for max_tokens) and are dropped
   const int valid = *valid_tokens;
-  const int row = row0 + g.lane / G;
-  if ((g.lane % G) == 0 && row < n_rows) {
 #pragma unroll
-    for (int t = 0; t < TC; ++t) {
-      float v = NM == 2 ? silu_f(tot[0][t]) * tot[NM - 1][t] : 1.0f * tot[0][t];
-      if (NM == 1 && bias) v += bias[row];
-      if (token0 + t < valid) out[t][row] = v;
+  for (int d = 0; d < D; ++d) {
+    float tot[NM][TC];
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+#pragma unroll
+      for (int t = 0; t < TC; ++t) tot[m][t] = 0.0f;
+      accum<QUANT, TC>(r[d][m], g, x, xs, tot[m]);
+#pragma unroll
+      for (int t = 0; t < TC; ++t) tot[m][t] = group_sum<G>(tot[m][t]);
+    }
+    const int row = row0 + d * RPS + g.lane / G;
+    if ((g.lane % G) == 0 && row < n_rows) {
+#pragma unroll
+      for (int t = 0; t < TC; ++t) {
+        float v = NM == 2 ? silu_f(tot[0][t]) * tot[NM - 1][t] : 1.0f * tot[0][t];
+        if (NM == 1 && bias) v += bias[row];
+        if (token0 + t < valid) out[t][row] = v;
+      }
     }
   }
 }
@@ -152,7 +165,7 @@ __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, cons
 // A: grid = max_tokens (norm + gate scalar) + chunks * tiles_r (router) + chunks * tiles_s (shared gate/up).
 // A chunk is two tokens sharing one pass over the weights.
 // ------------------------------------------------------------------------------------------------
-template <int SQ, int RF, int RPS>
+template <int SQ, int RF, int RPS, int kLogitsDepth>
 __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
   __shared__ float s_red[4];
   const int chunks = (a.max_tokens + 1) / 2;
@@ -165,25 +178,25 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
     if (!router) item -= n_r;
     const int tiles = router ? a.tiles_r : a.tiles_s;
     const int c = item / tiles, tile = item % tiles, t0 = 2 * c;
-    const int row0 = (tile * kWavesPerWg + wave) * RPS;
+    const int row0 = (tile * kWavesPerWg + wave) * RPS * kLogitsDepth;
     const float* x0 = a.residual + (size_t)t0 * a.H;
     if (t0 + 1 < a.max_tokens) {
       const float* const xr[2] = {x0, x0 + a.H};
       if (router) {
         float* const o[2] = {a.logits + (size_t)t0 * a.E, a.logits + (size_t)(t0 + 1) * a.E};
-        step_normed<RF, RPS, 2, 1>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0);
+        step_normed<RF, RPS, 2, 1, kLogitsDepth>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0);
       } else {
         float* const o[2] = {a.shared_inter + (size_t)t0 * a.I, a.shared_inter + (size_t)(t0 + 1) * a.I};
-        step_normed<SQ, RPS, 2, 2>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0);
+        step_normed<SQ, RPS, 2, 2, kLogitsDepth>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0);
       }
     } else {
       const float* const xr[1] = {x0};
       if (router) {
         float* const o[1] = {a.logits + (size_t)t0 * a.E};
-        step_normed<RF, RPS, 1, 1>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0);
+        step_normed<RF, RPS, 1, 1, kLogitsDepth>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0);
       } else {
         float* const o[1] = {a.shared_inter + (size_t)t0 * a.I};
-        step_normed<SQ, RPS, 1, 2>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0);
+        step_normed<SQ, RPS, 1, 2, kLogitsDepth>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0);
       }
     }
     XABE_TRACE(0, 3);
@@ -441,7 +454,13 @@ static bool launch_all(const Launch& l, int gq, int dq, int sgq, int sdq, int ro
   const bool rf32 = router_quant < 0;
   if (!rf32 && router_quant != XABE_QUANT_Q8_0) return false;
   if (l.launches & 1u) {
-#define XABE_A(SQ, RF) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH>), dim3(l.grid_a), dim3(256), 0, l.s, l.a)
+#define XABE_A(SQ, RF)                                                                                              \
+  do {                                                                                                            \
+    const int da = logits_depth(l.a.max_tokens);                                                                  \
+    if (da == 1) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 1>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);  \
+    else if (da == 2) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 2>), dim3(l.grid_a), dim3(256), 0, l.s, l.a); \
+    else hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 4>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);          \
+  } while (0)
     if (sg6 && rf32) XABE_A(kQ6K, kF32);
     else if (sg6) XABE_A(kQ6K, kQ8_0);
     else if (rf32) XABE_A(kQ8_0, kF32);
@@ -520,8 +539,9 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
   a.top_k = (int)g.experts_per_token;
   a.max_tokens = (int)g.max_tokens;
   const int rps_h = 2048 / a.H, rps_i = 2048 / a.I;
-  a.tiles_r = (a.E + kWavesPerWg * rps_h - 1) / (kWavesPerWg * rps_h);
-  a.tiles_s = (a.I + kWavesPerWg * rps_h - 1) / (kWavesPerWg * rps_h);
+  const int da = logits_depth(a.max_tokens);
+  a.tiles_r = (a.E + kWavesPerWg * rps_h * da - 1) / (kWavesPerWg * rps_h * da);
+  a.tiles_s = (a.I + kWavesPerWg * rps_h * da - 1) / (kWavesPerWg * rps_h * da);
   const int depth = a.H == 2048 ? 4 : 1;  // steps per wavefront of the gate/up launch (launch_shape)
   a.tiles_g = (a.I + kWavesPerWg * depth * rps_h - 1) / (kWavesPerWg * depth * rps_h);
   a.tiles_d = (a.H + kWavesPerWg * rps_i - 1) / (kWavesPerWg * rps_i);
