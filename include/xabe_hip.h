@@ -251,7 +251,7 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
                            size_t ffn_out_len, float* l_out, size_t l_out_len);
 int xabe_moe_block_disable_tensor_cores(xabe_moe_block* blk);            /* B:987-989 */
 int xabe_moe_block_set_exact_decode_regime(xabe_moe_block* blk, int on); /* B:1003-1005 */
-/* At max_tokens <= 16 and the model shapes (hidden 2048 / intermediate 512, and the 512 / 256 test shape) the
+/* At max_tokens <= 32 and the model shapes (hidden 2048 / intermediate 512, and the 512 / 256 test shape) the
  * block's eight steps are regrouped into three launches (logits + shared gate/up; route + gate/up; down +
  * combine) that compute the same values bit for bit.  `on` = 0 keeps one launch per step as the reference
  * has them (B:1091-1329); the switch exists for tests and measurement. */

@@ -1,4 +1,4 @@
-// The decode-width MoE block (max_tokens <= 16) as three launches with no intermediate passes.
+// The decode-width MoE block (max_tokens <= 32) as three launches with no intermediate passes.
 //
 // At a few tokens the block moves ~20 MB per token and every dependent memory access costs 1-2 us, so what
 // decides the time is the number of dependent round trips and launch boundaries on the critical path, not
@@ -37,7 +37,7 @@ namespace xabe { static __device__ long long g_route_trace[4096 * 8]; }
 
 namespace xabe {
 
-constexpr size_t kDecodeBlockMaxTokens = 16;  // widest batch served by the three launches (the dispatch-table regime is faster from ~24 tokens)
+constexpr size_t kDecodeBlockMaxTokens = 32;  // widest batch served by the three launches (at 32 tokens 198 against the dispatch-table regime's 203 us; it wins beyond)
 constexpr int kMaxTopK = 8;       // contributions held in registers by k_decode_down
 constexpr int kMaxInter = 512;    // intermediate width staged in LDS by k_decode_down
 // Steps per wavefront of the first launch: a wavefront reads 24 KB of activation rows and norm weights for the 2-4 KB

@@ -28,7 +28,7 @@ def _shift_layer(torch, X, w, off, which=None):
                              q("shared_up", w.shared_up), q("shared_down", w.shared_down))
 
 
-REGIMES = [(3, 3), (12, 11), (32, 29), (128, 100)]   # decode block (two format mixes), dispatch table, matrix cores
+REGIMES = [(3, 3), (12, 11), (32, 29), (40, 37), (128, 100)]   # decode block (two format mixes, widest), dispatch table, matrix cores
 
 
 def _layer(oracle, X, max_tokens):

@@ -259,7 +259,7 @@ def test_fused_shared_is_bit_identical_to_separate_launches(oracle, X, max_token
     assert torch.all(sh8 == 0)
 
 
-@pytest.mark.parametrize("geom,max_tokens,tokens", [("model", 8, 8), ("model", 32, 29), ("small", 40, 40), ("small", 5, 5)])
+@pytest.mark.parametrize("geom,max_tokens,tokens", [("model", 8, 8), ("model", 32, 29), ("model", 40, 37), ("small", 40, 40), ("small", 5, 5)])
 def test_weights_resident_dispatch_kernel_equals_the_plain_one(oracle, X, geom, max_tokens, tokens):
     # the dispatch-table regime (up to 63 tokens) keeps a tile's weights in registers across the block's token
     # chunks; force_community selects the plain per-chunk kernel: same bits, both stages

@@ -1,4 +1,4 @@
-"""The decode-width block (max_tokens <= 16) regrouped into three launches against the same block with one
+"""The decode-width block (max_tokens <= 32) regrouped into three launches against the same block with one
 launch per step (flat per-pair kernels up to 4 tokens, the dispatch-table regime above): every observable
 tensor bit for bit, over repeated calls, with fewer live tokens than
 the buffer holds, with and without a logit bias, and for each format pairing.  The per-step launches are
@@ -57,7 +57,8 @@ def _compare(X, oracle, g, tokens_seq, seed, router_q8=True, bias=False, expert_
 
 
 @pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (2, (2, 1, 2)), (3, (3, 1, 2, 3)), (4, (4, 3, 0, 4, 1)),
-                                                   (5, (5, 2, 5)), (8, (8, 1, 7)), (16, (16, 9, 0, 16))])
+                                                   (5, (5, 2, 5)), (8, (8, 1, 7)), (16, (16, 9, 0, 16)),
+                                                   (27, (27, 19)), (32, (32, 1, 32))])
 @pytest.mark.parametrize("router_q8", [True, False])
 def test_small_geometry(oracle, X, max_tokens, tokens_seq, router_q8):
     g = X.MoeGeometry(8, 2, 512, 256, 32, max_tokens)
@@ -91,7 +92,8 @@ def test_model_geometry_shipped_layout(oracle, X):
     blk.forward_stage(layer.dev, x, f, l, 2)
 
 
-@pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (3, (3, 3, 2)), (4, (4, 1, 4)), (7, (7, 5)), (16, (16, 11))])
+@pytest.mark.parametrize("max_tokens,tokens_seq", [(1, (1, 1)), (3, (3, 3, 2)), (4, (4, 1, 4)), (7, (7, 5)), (16, (16, 11)),
+                                                   (24, (24, 17)), (32, (32, 29))])
 def test_model_geometry(oracle, X, max_tokens, tokens_seq):
     g = X.MoeGeometry.qwen3_6(X.moe_block_size(max_tokens), max_tokens)
     _compare(X, oracle, g, tokens_seq, seed=4300 + max_tokens, bias=(max_tokens == 3))
