@@ -511,6 +511,10 @@ static int alloc_buffers(const xabe_moe_kernels* k, void* stream, int scope, boo
   A(&b->shared_inter_h, (wide && mma) ? g.max_tokens * g.intermediate : 0);
   b->n_tile_list = (wide && mma && routed) ? 4 * (eb + 1) + 4 : 0;
   A(&b->tile_list, b->n_tile_list);
+  b->n_router_partial = (mma && routed && g.max_tokens >= kRouterGemmMinTokens && router_gemm_splits(g) > 1)
+                            ? (size_t)router_gemm_splits(g) * g.max_tokens * g.num_experts
+                            : 0;
+  A(&b->router_partial, b->n_router_partial);
   b->bytes = total;
   b->valid_published = 0;
   if (st != XABE_OK) {
@@ -531,7 +535,7 @@ void xabe_moe_buffers_free(xabe_moe_buffers* b) {
   if (!b) return;
   void* ptrs[] = {b->topk_ids, b->topk_weights, b->sorted_token_ids, b->expert_ids, b->bucket_live, b->expert_counts,
                   b->num_tokens_post_pad, b->valid_tokens, b->align_hist, b->inter, b->partial, b->shared_inter, b->x_h, b->inter_h,
-                  b->shared_inter_h, b->tile_list};
+                  b->shared_inter_h, b->tile_list, b->router_partial};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   delete b;
@@ -921,7 +925,7 @@ int xabe_moe_router_logits(const xabe_moe_kernels* k, void* stream, const xabe_m
   }
   XABE_TRY(check_len("normed", g.max_tokens * g.hidden, normed_len));
   XABE_TRY(check_len("logits", g.max_tokens * g.num_experts, logits_len));
-  if (router_gemm_supported(k, fmt)) return launch_router_gemm(k, as_stream(stream), b, router, fmt, normed, logits);
+  if (router_gemm_supported(k, b, fmt)) return launch_router_gemm(k, as_stream(stream), b, router, fmt, normed, logits);
   ExpertArgs a = base_args(k, b);
   a.w0 = static_cast<const uint8_t*>(router);
   a.x = normed;

@@ -70,7 +70,17 @@ int dense_fp32_fused(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers*
                      xabe_quant_tensor up, xabe_quant_tensor down, const float* post_norm, float eps,
                      const float* residual, float* normed, float* ffn_out, float* l_out, bool* launched);
 // router logits as an fp32 matrix-core GEMM at prefill widths (router_gemm.hip)
-bool router_gemm_supported(const xabe_moe_kernels* k, int router_quant);
+// The router GEMM from kRouterGemmMinTokens up (below it the vector kernel), its contraction split over workgroups
+// while its 64-token x 128-expert tiles are fewer than the chip's 256 CUs: 8 parts up to 1024 tokens, 4 at 2048,
+// 2 at 4096, unsplit from 8192.
+constexpr size_t kRouterGemmMinTokens = 256;
+inline int router_gemm_splits(const xabe_moe_geometry& g) {
+  const size_t tiles = (g.num_experts / 128) * ((g.max_tokens + 63) / 64);
+  int splits = 1;
+  while (splits < 8 && tiles * splits < 256 && g.hidden % (size_t)(32 * splits * 2) == 0) splits *= 2;
+  return splits;
+}
+bool router_gemm_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int router_quant);
 int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,
                        int router_quant, const float* normed, float* logits);
 // one-time, at handle creation: LDS limits of the kernels that ask for more than the static 64 KB (mfma.hip, api.hip)
@@ -123,5 +133,7 @@ struct xabe_moe_buffers {
   uint16_t* shared_inter_h;
   int32_t* tile_list;   // device-built tile schedule
   size_t n_tile_list;
+  float* router_partial;  // [split][token][expert]: the router GEMM's contraction splits at mid widths
+  size_t n_router_partial;
   size_t bytes;
 };

@@ -8,6 +8,10 @@
 // value); products and sums are fp32 inside the matrix core.  The contraction order differs from the
 // decode kernels', so these logits agree with theirs to fp32 rounding, not bit for bit: as with the expert
 // contractions, a token is bit-identical across batches WITHIN a regime.
+// Below 8192 tokens the tiles are too few to fill the chip (8 x 2 at 512 tokens, each walking all 64 contraction
+// steps: ~115 us whatever the width), so the contraction is split over workgroups (grid.z: 8 parts up to 1024
+// tokens, 4 at 2048, 2 at 4096), each part writing its own [token][expert] plane, and a second small launch adds
+// the planes in part order: a fixed order, so a token's logits do not depend on its batch mates here either.
 // Replaces the reference's router launch for wide passes (crates/xabe-engine/src/block/moe.rs:1150-1184).
 #include <string.h>
 
@@ -27,12 +31,13 @@ constexpr int kRgLdB = kRgN + 1;
 struct RouterGemmArgs {
   const void* router;   // [E][H] f32, or Q8_0 blocks
   const float* normed;  // [T][H]
-  float* logits;        // [T][E]
+  float* logits;        // [T][E]; with splits > 1 the planes [split][max_tokens][E]
   const int* valid_tokens;
   int H, E;
+  int splits, max_tokens;
 };
 
-// grid: (E / 128, ceil(max_tokens / 64)); 4 wavefronts as 2 (tokens) x 2 (experts), each 32 x 64.
+// grid: (E / 128, ceil(max_tokens / 64), splits); 4 wavefronts as 2 (tokens) x 2 (experts), each 32 x 64.
 template <bool Q8>
 __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
   __shared__ float sA[kRgK * kRgLdA];
@@ -55,7 +60,8 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
 #pragma unroll
   for (int j = 0; j < 2; ++j) acc[j] = (float16v)(0.0f);
 
-  const int nks = a.H / kRgK;
+  const int nks_all = a.H / kRgK, ks0 = (int)blockIdx.z * (nks_all / a.splits), nks = ks0 + nks_all / a.splits;
+  float* const plane = a.logits + (size_t)blockIdx.z * a.max_tokens * a.E;
   float4 ra[2];
   float rb[16];
   auto load_step = [&](int ks) {
@@ -81,8 +87,8 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
       }
     }
   };
-  load_step(0);
-  for (int ks = 0; ks < nks; ++ks) {
+  load_step(ks0);
+  for (int ks = ks0; ks < nks; ++ks) {
     __syncthreads();  // the previous step's tiles have been read
     const float va[8] = {ra[0].x, ra[0].y, ra[0].z, ra[0].w, ra[1].x, ra[1].y, ra[1].z, ra[1].w};
 #pragma unroll
@@ -108,15 +114,29 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
     const int t = m0 + wm * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
     if (t >= valid) continue;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) a.logits[(size_t)t * a.E + n0 + wn * 64 + j * 32 + (lane & 31)] = acc[j][v];
+    for (int j = 0; j < 2; ++j) plane[(size_t)t * a.E + n0 + wn * 64 + j * 32 + (lane & 31)] = acc[j][v];
   }
 }
 
-bool router_gemm_supported(const xabe_moe_kernels* k, int router_quant) {
+// logits[t][e] = planes[0][t][e] + planes[1][t][e] + ... in part order, live tokens only
+__global__ void __launch_bounds__(256) k_router_sum_planes(const float* __restrict__ planes, const int* __restrict__ valid_tokens,
+                                                            int splits, int max_tokens, int E, float* __restrict__ logits) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)*valid_tokens * E) return;
+  float s = planes[i];
+  for (int z = 1; z < splits; ++z) s += planes[(size_t)z * max_tokens * E + i];
+  logits[i] = s;
+}
+
+bool router_gemm_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int router_quant) {
   const xabe_moe_geometry& g = k->g;
-  // below ~2048 tokens the 64 x 128 tiles are too few to fill the chip and the decode-style kernel wins
-  if (!k->tensor_cores || k->exact_regime || k->force_community || g.max_tokens < 2048) return false;
+  // below 256 tokens even the split tiles are too few and the decode-style kernel wins
+  if (!k->tensor_cores || k->exact_regime || k->force_community || g.max_tokens < kRouterGemmMinTokens) return false;
   if (!(router_quant < 0 || router_quant == XABE_QUANT_Q8_0)) return false;
+  const int splits = router_gemm_splits(g);
+  if (splits > 1 && (!b->router_partial || b->n_router_partial < (size_t)splits * g.max_tokens * g.num_experts ||
+                     g.hidden % (kRgK * splits) != 0))
+    return false;
   return g.hidden % kRgK == 0 && g.num_experts % kRgN == 0;
 }
 
@@ -125,16 +145,24 @@ int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_
   const xabe_moe_geometry& g = k->g;
   RouterGemmArgs a;
   memset(&a, 0, sizeof(a));
+  a.splits = router_gemm_splits(g);
+  a.max_tokens = (int)g.max_tokens;
   a.router = router;
   a.normed = normed;
-  a.logits = logits;
+  a.logits = a.splits > 1 ? b->router_partial : logits;
   a.valid_tokens = b->valid_tokens;
   a.H = (int)g.hidden;
   a.E = (int)g.num_experts;
-  dim3 grid((unsigned)(g.num_experts / kRgN), (unsigned)((g.max_tokens + kRgM - 1) / kRgM));
+  dim3 grid((unsigned)(g.num_experts / kRgN), (unsigned)((g.max_tokens + kRgM - 1) / kRgM), (unsigned)a.splits);
   if (router_quant < 0) hipLaunchKernelGGL(k_router_gemm<false>, grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL(k_router_gemm<true>, grid, dim3(256), 0, s, a);
   XABE_HIP_TRY(hipGetLastError());
+  if (a.splits > 1) {
+    const size_t n = g.max_tokens * g.num_experts;
+    hipLaunchKernelGGL(k_router_sum_planes, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, b->router_partial,
+                       b->valid_tokens, a.splits, a.max_tokens, a.E, logits);
+    XABE_HIP_TRY(hipGetLastError());
+  }
   return XABE_OK;
 }
 
