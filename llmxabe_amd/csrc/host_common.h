@@ -71,13 +71,13 @@ int dense_fp32_fused(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers*
                      const float* residual, float* normed, float* ffn_out, float* l_out, bool* launched);
 // router logits as an fp32 matrix-core GEMM at prefill widths (router_gemm.hip)
 // The router GEMM from kRouterGemmMinTokens up (below it the vector kernel), its contraction split over workgroups
-// while its 64-token x 128-expert tiles are fewer than the chip's 256 CUs: 8 parts up to 1024 tokens, 4 at 2048,
-// 2 at 4096, unsplit from 8192.
+// while its 64-token x 128-expert tiles are fewer than four per CU: 8 parts up to 4096 tokens, 4 at 8192, 2 at
+// 16384, unsplit beyond.
 constexpr size_t kRouterGemmMinTokens = 256;
 inline int router_gemm_splits(const xabe_moe_geometry& g) {
   const size_t tiles = (g.num_experts / 128) * ((g.max_tokens + 63) / 64);
   int splits = 1;
-  while (splits < 8 && tiles * splits < 256 && g.hidden % (size_t)(32 * splits * 2) == 0) splits *= 2;
+  while (splits < 8 && tiles * splits < 1024 && g.hidden % (size_t)(32 * splits * 2) == 0) splits *= 2;
   return splits;
 }
 bool router_gemm_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int router_quant);

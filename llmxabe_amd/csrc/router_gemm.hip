@@ -8,10 +8,11 @@
 // value); products and sums are fp32 inside the matrix core.  The contraction order differs from the
 // decode kernels', so these logits agree with theirs to fp32 rounding, not bit for bit: as with the expert
 // contractions, a token is bit-identical across batches WITHIN a regime.
-// Below 8192 tokens the tiles are too few to fill the chip (8 x 2 at 512 tokens, each walking all 64 contraction
-// steps: ~115 us whatever the width), so the contraction is split over workgroups (grid.z: 8 parts up to 1024
-// tokens, 4 at 2048, 2 at 4096), each part writing its own [token][expert] plane, and a second small launch adds
-// the planes in part order: a fixed order, so a token's logits do not depend on its batch mates here either.
+// Up to 16384 tokens the tiles are too few to fill the chip with more than a workgroup or two per CU (8 x 2 at
+// 512 tokens, each walking all 64 contraction steps: ~115 us whatever the width), so the contraction is split
+// over workgroups (grid.z: 8 parts up to 4096 tokens, 4 at 8192), each part writing its own [token][expert] plane,
+// and a second small launch adds the planes in part order: a fixed order, so a token's logits do not depend on
+// its batch mates here either.
 // Replaces the reference's router launch for wide passes (crates/xabe-engine/src/block/moe.rs:1150-1184).
 #include <string.h>
 
