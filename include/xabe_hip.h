@@ -286,7 +286,45 @@ int xabe_dense_ffn_block_forward(xabe_dense_ffn_block* blk, void* stream, const 
                                  const float* residual, size_t residual_len, size_t tokens, float* ffn_out,
                                  size_t ffn_out_len, float* l_out, size_t l_out_len);
 int xabe_dense_ffn_block_disable_tensor_cores(xabe_dense_ffn_block* blk);
+int xabe_dense_ffn_block_tensor_cores_enabled(const xabe_dense_ffn_block* blk);
+int xabe_dense_ffn_block_publish_tokens(xabe_dense_ffn_block* blk, void* stream, size_t tokens); /* D: publish_tokens */
 const float* xabe_dense_ffn_block_normed(const xabe_dense_ffn_block* blk, size_t* len);
+
+/* ---- FfnBlock / FfnLayerWeights (crates/xabe-engine/src/block/ffn.rs:27-228): which feed-forward block a layer
+ * runs, chosen once from the model configuration; the pairing of block and weights is checked on every pass. ---- */
+typedef enum xabe_ffn_kind { XABE_FFN_MOE = 0, XABE_FFN_DENSE = 1 } xabe_ffn_kind;
+/* The fields of ModelConfig the geometry is made from (crates/xabe-model/src/config.rs:126-187): `hidden` for both
+ * kinds; the MoeConfig fields for XABE_FFN_MOE, DenseFfnConfig::intermediate for XABE_FFN_DENSE. */
+typedef struct xabe_ffn_config {
+  int kind; /* xabe_ffn_kind */
+  size_t hidden;
+  size_t num_experts, experts_per_token, expert_intermediate;
+  size_t dense_intermediate;
+} xabe_ffn_config;
+typedef struct xabe_ffn_layer_weights {
+  int kind; /* xabe_ffn_kind: which of the two members below is filled in */
+  xabe_moe_layer_weights moe;
+  xabe_dense_ffn_layer_weights dense;
+} xabe_ffn_layer_weights;
+typedef struct xabe_ffn_block xabe_ffn_block;
+/* FfnBlock::geometry_for (ffn.rs:92-104): dense = one expert, top-1, at the MLP's intermediate width. */
+int xabe_ffn_block_geometry_for(const xabe_ffn_config* config, size_t block_size, size_t max_tokens, xabe_moe_geometry* out);
+/* FfnBlock::new (ffn.rs:107-127) */
+int xabe_ffn_block_new(const xabe_ffn_config* config, const xabe_moe_geometry* geometry, float eps, void* stream,
+                       xabe_ffn_block** out);
+void xabe_ffn_block_free(xabe_ffn_block* blk);
+int xabe_ffn_block_kind(const xabe_ffn_block* blk);
+int xabe_ffn_block_disable_tensor_cores(xabe_ffn_block* blk);            /* ffn.rs:130-135 */
+int xabe_ffn_block_tensor_cores_enabled(const xabe_ffn_block* blk);      /* ffn.rs:138-143 */
+int xabe_ffn_block_set_exact_decode_regime(xabe_ffn_block* blk, int on); /* ffn.rs:148-152: a no-op on the dense block */
+int xabe_ffn_block_geometry(const xabe_ffn_block* blk, xabe_moe_geometry* out); /* ffn.rs:155-160 */
+const float* xabe_ffn_block_normed(const xabe_ffn_block* blk, size_t* len);     /* ffn.rs:163-168 */
+xabe_moe_block* xabe_ffn_block_as_moe(const xabe_ffn_block* blk);               /* ffn.rs:173-178: NULL on the dense path */
+int xabe_ffn_block_publish_tokens(xabe_ffn_block* blk, void* stream, size_t tokens); /* ffn.rs:182-191 */
+/* FfnBlock::forward (ffn.rs:199-212): XABE_ERR_FFN_KIND_MISMATCH, nothing launched, when block and weights differ in kind. */
+int xabe_ffn_block_forward(xabe_ffn_block* blk, void* stream, const xabe_ffn_layer_weights* w, const float* residual,
+                           size_t residual_len, size_t tokens, float* ffn_out, size_t ffn_out_len, float* l_out,
+                           size_t l_out_len);
 
 /* ---- synthetic stacks for benches (the role of crates/xabe-cuda/src/bin/bench_moe.rs:140-334) ----
  * Fills device memory with seeded values: element i belongs to chunk i/256, chunk c draws from

@@ -2,6 +2,7 @@
 from .moe import (BLOCK_Q6_K_DEVICE_BYTES, BufferScope, ExpertQuant, LayerOpsKernels, MoeBuffers, MoeError,  # noqa: F401
                   MoeGeometry, MoeKernels, QuantTensor, calibrate_hbm_read, calibrate_mfma_f16, dequantize, moe_block_size,
                   synth_normal_f32, synth_quant, to_device_layout)
-from .block import DEFAULT_RMS_EPS, DenseFfnBlock, DenseFfnLayerWeights, MoeBlock, MoeLayerWeights  # noqa: F401
+from .block import (DEFAULT_RMS_EPS, DenseFfnBlock, DenseFfnLayerWeights, FfnBlock, FfnConfig, FfnKind,  # noqa: F401
+                    FfnLayerWeights, MoeBlock, MoeLayerWeights)
 from .gguf import GgmlType, GgufError, GgufFile, TensorInfo, UploadedDenseFfnLayer, UploadedMoeLayer  # noqa: F401
 from .lm_head import ARGMAX_BLOCKS, MAX_BATCH_TILE, HeadFormat, HeadTensor, LmHeadGeometry, LmHeadKernels  # noqa: F401

@@ -38,6 +38,15 @@ class DenseLayerWeightsC(C.Structure):
     _fields_ = [("post_norm", vp), ("gate", QuantTensorC), ("up", QuantTensorC), ("down", QuantTensorC)]
 
 
+class FfnConfigC(C.Structure):
+    _fields_ = [("kind", C.c_int), ("hidden", sz), ("num_experts", sz), ("experts_per_token", sz),
+                ("expert_intermediate", sz), ("dense_intermediate", sz)]
+
+
+class FfnLayerWeightsC(C.Structure):
+    _fields_ = [("kind", C.c_int), ("moe", MoeLayerWeightsC), ("dense", DenseLayerWeightsC)]
+
+
 class LmHeadGeometryC(C.Structure):
     _fields_ = [("hidden", sz), ("vocab", sz), ("max_tokens", sz)]
 
@@ -123,6 +132,20 @@ _SIGNATURES = {
     "xabe_dense_ffn_block_forward": (C.c_int, [vp, vp, C.POINTER(DenseLayerWeightsC), vp, sz, sz, vp, sz, vp, sz]),
     "xabe_dense_ffn_block_disable_tensor_cores": (C.c_int, [vp]),
     "xabe_dense_ffn_block_normed": (vp, [vp, C.POINTER(sz)]),
+    "xabe_dense_ffn_block_tensor_cores_enabled": (C.c_int, [vp]),
+    "xabe_dense_ffn_block_publish_tokens": (C.c_int, [vp, vp, sz]),
+    "xabe_ffn_block_geometry_for": (C.c_int, [C.POINTER(FfnConfigC), sz, sz, C.POINTER(Geometry)]),
+    "xabe_ffn_block_new": (C.c_int, [C.POINTER(FfnConfigC), C.POINTER(Geometry), C.c_float, vp, C.POINTER(vp)]),
+    "xabe_ffn_block_free": (None, [vp]),
+    "xabe_ffn_block_kind": (C.c_int, [vp]),
+    "xabe_ffn_block_disable_tensor_cores": (C.c_int, [vp]),
+    "xabe_ffn_block_tensor_cores_enabled": (C.c_int, [vp]),
+    "xabe_ffn_block_set_exact_decode_regime": (C.c_int, [vp, C.c_int]),
+    "xabe_ffn_block_geometry": (C.c_int, [vp, C.POINTER(Geometry)]),
+    "xabe_ffn_block_normed": (vp, [vp, C.POINTER(sz)]),
+    "xabe_ffn_block_as_moe": (vp, [vp]),
+    "xabe_ffn_block_publish_tokens": (C.c_int, [vp, vp, sz]),
+    "xabe_ffn_block_forward": (C.c_int, [vp, vp, C.POINTER(FfnLayerWeightsC), vp, sz, sz, vp, sz, vp, sz]),
     "xabe_synth_normal_f32": (C.c_int, [vp, C.c_uint64, sz, C.c_float, vp]),
     "xabe_calibrate_hbm_read": (C.c_int, [vp, vp, sz, vp]),
     "xabe_calibrate_mfma_f16": (C.c_int, [vp, vp, sz, C.c_int, C.POINTER(C.c_double)]),

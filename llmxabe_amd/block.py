@@ -1,16 +1,18 @@
 """Block-level mirrors of `MoeBlock` / `MoeLayerWeights` (crates/xabe-engine/src/block/moe.rs:634-1330)
-and `DenseFfnBlock` (crates/xabe-engine/src/block/dense_ffn.rs).  The sequencing itself lives in the
+`DenseFfnBlock` (crates/xabe-engine/src/block/dense_ffn.rs) and `FfnBlock` (crates/xabe-engine/src/block/ffn.rs).
+The sequencing itself lives in the
 library (csrc/block.hip); these classes hold the handles and the device tensors."""
 from __future__ import annotations
 
 import ctypes as C
+import enum
 from dataclasses import dataclass
 from typing import Optional
 
 import torch
 
 from . import _ffi
-from ._ffi import DenseLayerWeightsC, MoeLayerWeightsC
+from ._ffi import DenseLayerWeightsC, FfnConfigC, FfnLayerWeightsC, Geometry, MoeLayerWeightsC
 from .moe import ExpertQuant, MoeBuffers, MoeGeometry, QuantTensor, _ptr, _stream, _wrap, check
 
 DEFAULT_RMS_EPS = 1e-6  # block/moe.rs:179
@@ -130,3 +132,125 @@ class DenseFfnBlock:
         n = C.c_size_t(0)
         p = _ffi.lib().xabe_dense_ffn_block_normed(self._h, C.byref(n))
         return _wrap(p, n.value, torch.float32)
+
+    def publish_tokens(self, tokens: int):
+        check(_ffi.lib().xabe_dense_ffn_block_publish_tokens(self._h, _stream(), tokens))
+
+    def tensor_cores_enabled(self) -> bool:
+        return bool(_ffi.lib().xabe_dense_ffn_block_tensor_cores_enabled(self._h))
+
+
+class FfnKind(enum.IntEnum):
+    MOE = 0
+    DENSE = 1
+
+
+@dataclass
+class FfnConfig:
+    """The fields of `ModelConfig` the feed-forward geometry is made from
+    (crates/xabe-model/src/config.rs:126-187)."""
+    kind: FfnKind
+    hidden: int
+    num_experts: int = 0
+    experts_per_token: int = 0
+    expert_intermediate: int = 0
+    dense_intermediate: int = 0
+
+    @staticmethod
+    def qwen3_6_35b_a3b() -> "FfnConfig":
+        return FfnConfig(FfnKind.MOE, 2048, 256, 8, 512, 0)
+
+    @staticmethod
+    def qwen3_8_27b() -> "FfnConfig":
+        return FfnConfig(FfnKind.DENSE, 5120, 0, 0, 0, 17408)
+
+    def _c(self) -> FfnConfigC:
+        return FfnConfigC(int(self.kind), self.hidden, self.num_experts, self.experts_per_token,
+                          self.expert_intermediate, self.dense_intermediate)
+
+
+class FfnLayerWeights:
+    """`FfnLayerWeights` (crates/xabe-engine/src/block/ffn.rs:43-48): one layer's weights, either kind."""
+
+    def __init__(self, w):
+        if isinstance(w, MoeLayerWeights):
+            self.kind = FfnKind.MOE
+        elif isinstance(w, DenseFfnLayerWeights):
+            self.kind = FfnKind.DENSE
+        else:
+            raise TypeError("FfnLayerWeights wraps MoeLayerWeights or DenseFfnLayerWeights")
+        self.inner = w
+
+    def _c(self) -> FfnLayerWeightsC:
+        c = FfnLayerWeightsC()
+        c.kind = int(self.kind)
+        if self.kind == FfnKind.MOE:
+            c.moe = self.inner._c()
+        else:
+            c.dense = self.inner._c()
+        return c
+
+
+class FfnBlock:
+    """`FfnBlock` (crates/xabe-engine/src/block/ffn.rs:27-228): the feed-forward block of one pass shape,
+    MoE or dense, chosen once from the configuration."""
+
+    @staticmethod
+    def geometry_for(config: FfnConfig, block_size: int, max_tokens: int) -> MoeGeometry:
+        g = Geometry()
+        check(_ffi.lib().xabe_ffn_block_geometry_for(C.byref(config._c()), block_size, max_tokens, C.byref(g)))
+        return MoeGeometry(g.num_experts, g.experts_per_token, g.hidden, g.intermediate, g.block_size, g.max_tokens)
+
+    def __init__(self, config: FfnConfig, geometry: MoeGeometry, eps: float = DEFAULT_RMS_EPS):
+        h = C.c_void_p()
+        check(_ffi.lib().xabe_ffn_block_new(C.byref(config._c()), C.byref(geometry._c()), eps, _stream(), C.byref(h)))
+        self._h = h.value
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            try:
+                _ffi.lib().xabe_ffn_block_free(self._h)
+            except Exception:  # interpreter shutdown
+                pass
+            self._h = None
+
+    def kind(self) -> FfnKind: return FfnKind(_ffi.lib().xabe_ffn_block_kind(self._h))
+    def disable_tensor_cores(self): check(_ffi.lib().xabe_ffn_block_disable_tensor_cores(self._h))
+    def tensor_cores_enabled(self) -> bool: return bool(_ffi.lib().xabe_ffn_block_tensor_cores_enabled(self._h))
+    def set_exact_decode_regime(self, on: bool): check(_ffi.lib().xabe_ffn_block_set_exact_decode_regime(self._h, int(on)))
+
+    def geometry(self) -> MoeGeometry:
+        g = Geometry()
+        check(_ffi.lib().xabe_ffn_block_geometry(self._h, C.byref(g)))
+        return MoeGeometry(g.num_experts, g.experts_per_token, g.hidden, g.intermediate, g.block_size, g.max_tokens)
+
+    def normed(self) -> torch.Tensor:
+        n = C.c_size_t(0)
+        p = _ffi.lib().xabe_ffn_block_normed(self._h, C.byref(n))
+        return _wrap(p, n.value, torch.float32)
+
+    def as_moe(self) -> Optional[MoeBlock]:
+        """A borrowed view of the routed block, None on the dense path."""
+        p = _ffi.lib().xabe_ffn_block_as_moe(self._h)
+        return _BorrowedMoeBlock(p, self) if p else None
+
+    def publish_tokens(self, tokens: int):
+        check(_ffi.lib().xabe_ffn_block_publish_tokens(self._h, _stream(), tokens))
+
+    def forward(self, w: FfnLayerWeights, residual, tokens: int, ffn_out, l_out):
+        cw = w._c()
+        check(_ffi.lib().xabe_ffn_block_forward(self._h, _stream(), C.byref(cw), _ptr(residual), residual.numel(), tokens,
+                                                _ptr(ffn_out), ffn_out.numel(), _ptr(l_out), l_out.numel()))
+
+
+class _BorrowedMoeBlock(MoeBlock):
+    """A `MoeBlock` view over a handle another object owns (FfnBlock.as_moe)."""
+
+    def __init__(self, handle, owner):  # noqa: D401 - no allocation here
+        self._h = handle
+        self._owner = owner
+        self._geometry = owner.geometry()
+        self._eps = None
+
+    def __del__(self):
+        self._h = None

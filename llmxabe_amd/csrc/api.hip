@@ -565,10 +565,20 @@ int xabe_moe_set_valid_tokens(const xabe_moe_kernels* k, void* stream, xabe_moe_
     return set_error(XABE_ERR_TOO_MANY_TOKENS, "%zu tokens exceeds the %zu the buffers were sized for", tokens,
                      k->g.max_tokens);
   if (b->valid_published == (int32_t)tokens) return XABE_OK;
-  const int32_t v = (int32_t)tokens;
-  // pageable source: the copy is staged before the call returns, so `v` may go out of scope
-  XABE_HIP_TRY(hipMemcpyAsync(b->valid_tokens, &v, sizeof(v), hipMemcpyHostToDevice, as_stream(stream)));
-  b->valid_published = v;
+  // A change of the count is a host-to-device copy, and a copy recorded into a graph would publish, on every replay,
+  // whatever the source holds then.  Like the reference (kernels/moe.rs:5473-5491: "callable outside graph capture"),
+  // the count is set before a capture begins; a call that would change it inside one is refused, with nothing recorded.
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  XABE_HIP_TRY(hipStreamIsCapturing(as_stream(stream), &capturing));
+  if (capturing != hipStreamCaptureStatusNone)
+    return set_error(XABE_ERR_INVALID_ARGUMENT,
+                     "set_valid_tokens: the stream is capturing and the live-token count would change from %d to %zu; "
+                     "publish the count before the capture begins",
+                     (int)b->valid_published, tokens);
+  // the source is a slot the buffers own, so it outlives the copy however the runtime stages it
+  b->valid_host = (int32_t)tokens;
+  XABE_HIP_TRY(hipMemcpyAsync(b->valid_tokens, &b->valid_host, sizeof(b->valid_host), hipMemcpyHostToDevice, as_stream(stream)));
+  b->valid_published = b->valid_host;
   return XABE_OK;
 }
 

@@ -106,6 +106,8 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
   XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
                          g.hidden, blk->eps));
   // 2. router logits, (bias,) softmax + top-k + renormalise, dispatch tables
+  if (!(w->router_quant < 0 || w->router_quant == XABE_QUANT_Q8_0))
+    return set_error(XABE_ERR_UNSUPPORTED_QUANT, "router: only f32 and Q8_0 routers are supported, got code %d", w->router_quant);
   const size_t router_len = w->router_quant < 0
                                 ? g.num_experts * g.hidden
                                 : g.num_experts * g.hidden / xabe_expert_quant_block_elements(w->router_quant) *
@@ -256,4 +258,112 @@ int xabe_dense_ffn_block_forward(xabe_dense_ffn_block* blk, void* stream, const 
     XABE_TRY(xabe_moe_shared_expert(blk->moe, stream, blk->buffers, w->gate, w->up, w->down, blk->normed, blk->n_act,
                                     ffn_out, blk->n_act));
   return xabe_dense_ffn_add_residual(blk->moe, stream, blk->buffers, ffn_out, residual, l_out);
+}
+
+int xabe_dense_ffn_block_publish_tokens(xabe_dense_ffn_block* blk, void* stream, size_t tokens) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "publish_tokens: null handle");
+  return xabe_moe_set_valid_tokens(blk->moe, stream, blk->buffers, tokens);
+}
+int xabe_dense_ffn_block_tensor_cores_enabled(const xabe_dense_ffn_block* blk) {
+  return blk ? xabe_moe_kernels_tensor_cores_enabled(blk->moe) : 0;
+}
+
+// ------------------------------------------------------------------ FfnBlock
+// The two-variant dispatch of crates/xabe-engine/src/block/ffn.rs:27-228: one handle that is either block,
+// one weights value that is either layer kind, and a pairing that is checked rather than assumed.
+struct xabe_ffn_block {
+  int kind;
+  xabe_moe_block* moe;
+  xabe_dense_ffn_block* dense;
+};
+
+static const char* ffn_kind_name(int kind) { return kind == XABE_FFN_MOE ? "moe" : kind == XABE_FFN_DENSE ? "dense" : "unknown"; }
+
+int xabe_ffn_block_geometry_for(const xabe_ffn_config* config, size_t block_size, size_t max_tokens, xabe_moe_geometry* out) {
+  if (!config || !out) return set_error(XABE_ERR_INVALID_ARGUMENT, "FfnBlock::geometry_for: null pointer");
+  if (config->kind == XABE_FFN_MOE) {  // MoeBlock::geometry_for (block/moe.rs:931-945)
+    *out = {config->num_experts, config->experts_per_token, config->hidden, config->expert_intermediate, block_size, max_tokens};
+    return XABE_OK;
+  }
+  if (config->kind == XABE_FFN_DENSE) {  // DenseFfnBlock::geometry_for (block/dense_ffn.rs:836-850)
+    *out = {1, 1, config->hidden, config->dense_intermediate, block_size, max_tokens};
+    return XABE_OK;
+  }
+  return set_error(XABE_ERR_INVALID_ARGUMENT, "FfnBlock::geometry_for: unknown feed-forward kind %d", config->kind);
+}
+
+int xabe_ffn_block_new(const xabe_ffn_config* config, const xabe_moe_geometry* geometry, float eps, void* stream,
+                       xabe_ffn_block** out) {
+  if (!config || !geometry || !out) return set_error(XABE_ERR_INVALID_ARGUMENT, "FfnBlock::new: null pointer");
+  if (config->kind != XABE_FFN_MOE && config->kind != XABE_FFN_DENSE)
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "FfnBlock::new: unknown feed-forward kind %d", config->kind);
+  xabe_ffn_block* blk = new xabe_ffn_block();
+  blk->kind = config->kind;
+  blk->moe = nullptr;
+  blk->dense = nullptr;
+  const int st = config->kind == XABE_FFN_MOE
+                     ? xabe_moe_block_new(geometry, eps, stream, &blk->moe)
+                     : xabe_dense_ffn_block_new(geometry->hidden, geometry->intermediate, geometry->max_tokens, eps, stream,
+                                                &blk->dense);
+  if (st != XABE_OK) {
+    delete blk;
+    return st;
+  }
+  *out = blk;
+  return XABE_OK;
+}
+
+void xabe_ffn_block_free(xabe_ffn_block* blk) {
+  if (!blk) return;
+  xabe_moe_block_free(blk->moe);
+  xabe_dense_ffn_block_free(blk->dense);
+  delete blk;
+}
+
+int xabe_ffn_block_kind(const xabe_ffn_block* blk) { return blk ? blk->kind : -1; }
+
+int xabe_ffn_block_disable_tensor_cores(xabe_ffn_block* blk) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "disable_tensor_cores: null handle");
+  return blk->kind == XABE_FFN_MOE ? xabe_moe_block_disable_tensor_cores(blk->moe)
+                                   : xabe_dense_ffn_block_disable_tensor_cores(blk->dense);
+}
+int xabe_ffn_block_tensor_cores_enabled(const xabe_ffn_block* blk) {
+  if (!blk) return 0;
+  return blk->kind == XABE_FFN_MOE ? xabe_moe_block_tensor_cores_enabled(blk->moe)
+                                   : xabe_dense_ffn_block_tensor_cores_enabled(blk->dense);
+}
+int xabe_ffn_block_set_exact_decode_regime(xabe_ffn_block* blk, int on) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_exact_decode_regime: null handle");
+  // the dense block has no routed kernels and so no regime to pin (block/ffn.rs:146-153)
+  return blk->kind == XABE_FFN_MOE ? xabe_moe_block_set_exact_decode_regime(blk->moe, on) : XABE_OK;
+}
+int xabe_ffn_block_geometry(const xabe_ffn_block* blk, xabe_moe_geometry* out) {
+  if (!blk || !out) return set_error(XABE_ERR_INVALID_ARGUMENT, "geometry: null pointer");
+  *out = blk->kind == XABE_FFN_MOE ? blk->moe->g : blk->dense->g;
+  return XABE_OK;
+}
+const float* xabe_ffn_block_normed(const xabe_ffn_block* blk, size_t* len) {
+  if (!blk) { if (len) *len = 0; return nullptr; }
+  return blk->kind == XABE_FFN_MOE ? xabe_moe_block_normed(blk->moe, len) : xabe_dense_ffn_block_normed(blk->dense, len);
+}
+xabe_moe_block* xabe_ffn_block_as_moe(const xabe_ffn_block* blk) { return blk ? blk->moe : nullptr; }
+
+int xabe_ffn_block_publish_tokens(xabe_ffn_block* blk, void* stream, size_t tokens) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "publish_tokens: null handle");
+  return blk->kind == XABE_FFN_MOE ? xabe_moe_block_publish_tokens(blk->moe, stream, tokens)
+                                   : xabe_dense_ffn_block_publish_tokens(blk->dense, stream, tokens);
+}
+
+int xabe_ffn_block_forward(xabe_ffn_block* blk, void* stream, const xabe_ffn_layer_weights* w, const float* residual,
+                           size_t residual_len, size_t tokens, float* ffn_out, size_t ffn_out_len, float* l_out,
+                           size_t l_out_len) {
+  if (!blk || !w) return set_error(XABE_ERR_INVALID_ARGUMENT, "FfnBlock::forward: null pointer");
+  if (blk->kind != w->kind)  // checked before anything is launched (block/ffn.rs:205-208)
+    return set_error(XABE_ERR_FFN_KIND_MISMATCH, "a `%s` feed-forward block was handed `%s` weights", ffn_kind_name(blk->kind),
+                     ffn_kind_name(w->kind));
+  if (blk->kind == XABE_FFN_MOE)
+    return xabe_moe_block_forward(blk->moe, stream, &w->moe, residual, residual_len, tokens, nullptr, ffn_out, ffn_out_len,
+                                  l_out, l_out_len);
+  return xabe_dense_ffn_block_forward(blk->dense, stream, &w->dense, residual, residual_len, tokens, ffn_out, ffn_out_len,
+                                      l_out, l_out_len);
 }

@@ -122,7 +122,8 @@ struct xabe_moe_buffers {
   size_t n_align_chunks;
   int32_t* num_tokens_post_pad;
   int32_t* valid_tokens;
-  int32_t valid_published;
+  int32_t valid_published;  // what `valid_tokens` holds (0 after allocation)
+  int32_t valid_host;       // source of the host-to-device copy that publishes a new count
   float* inter;         // [slot][intermediate] fp32 (decode regimes)
   float* partial;       // [flat][hidden]
   float* shared_inter;  // [token][intermediate]

@@ -631,6 +631,7 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
   if (!k->tensor_cores || k->exact_regime || g.max_tokens < kMfmaMinTokens) return false;
   if (!b->x_h || !b->shared_inter_h) return false;
   if (routed && (!b->inter_h || !b->tile_list)) return false;
+  if (routed && g.num_experts > 512) return false;  // k_build_tiles scans two experts per thread of one 256-thread workgroup
   auto ok = [](int q) { return q == XABE_QUANT_Q6K || q == XABE_QUANT_Q8_0; };
   if (!ok(gate_q) || !ok(down_q) || gate_q != up_q) return false;
   // contraction in steps of 128 (whole Q6_K superblocks: 256); gate/up tiles 64 columns, down tiles 128

@@ -73,3 +73,17 @@ def test_errors_without_a_device_are_reported_not_crashed():
         X.MoeKernels(X.MoeGeometry(256, 8, 2048, 512, 0, 4))
     with pytest.raises(X.moe.UnsupportedGeometry, match="dispatch-block capacity exceeds the 65535 grid.y limit"):
         X.MoeKernels(X.MoeGeometry(512, 512, 2048, 512, 1, 65535))
+
+
+def test_ffn_block_geometry_for_each_architecture():
+    # crates/xabe-engine/src/block/ffn.rs:243-256: each architecture gets a geometry and they are not the same one
+    import llmxabe_amd as X
+
+    moe = X.FfnBlock.geometry_for(X.FfnConfig.qwen3_6_35b_a3b(), 32, 128)
+    dense = X.FfnBlock.geometry_for(X.FfnConfig.qwen3_8_27b(), 32, 128)
+    assert (moe.hidden, moe.intermediate, moe.num_experts) == (2048, 512, 256)
+    assert (dense.hidden, dense.intermediate, dense.num_experts) == (5120, 17408, 1)
+    assert (moe.experts_per_token, dense.experts_per_token) == (8, 1)
+    assert (moe.block_size, moe.max_tokens, dense.block_size, dense.max_tokens) == (32, 128, 32, 128)
+    with pytest.raises(X.moe.InvalidArgument, match="unknown feed-forward kind"):
+        X.FfnBlock.geometry_for(X.FfnConfig(7, 2048), 32, 128)

@@ -67,19 +67,8 @@ def test_grouped_forward_small_geometry(oracle, X, max_tokens, tokens, fmt):
     assert np.all(out[tokens:] == 0)  # rows past `tokens` are never written (moe_differential.rs:828-838)
 
 
-@pytest.mark.parametrize("max_tokens,tokens", [(1, 1), (3, 3), (4, 2), (32, 32), (37, 37)])
-def test_grouped_forward_model_geometry(oracle, X, max_tokens, tokens):
-    g = X.MoeGeometry.qwen3_6(32, max_tokens)
-    layer = make_layer(oracle, g, seed=500)
-    x = activations(12, max_tokens, 2048, tokens)
-    r = oracle.Xorshift64Star(0xA11 + tokens)
-    logits = np.stack([r.vec_f32(256, -8.0, 8.0) for _ in range(tokens)])
-    out, ids, w, _ = _grouped(X, oracle, g, layer, x, tokens, logits)
-    ref_ids, ref_w = oracle.route_batch(logits, 8)
-    assert np.array_equal(ids, ref_ids.astype(np.int32))
-    # naive_forward over the selected experts only (dequantise on demand)
-    host = layer.host
-    xs = x.cpu().numpy()
+def _naive_model_ref(oracle, host, xs, ref_ids, ref_w, tokens):
+    """naive_forward over the selected experts only (dequantised on demand), model geometry, Q6_K."""
     ref = np.zeros((tokens, 2048), np.float32)
     mat = 512 * 2048 // 256 * 210
     cache = {}
@@ -93,8 +82,47 @@ def test_grouped_forward_model_geometry(oracle, X, max_tokens, tokens):
             c = oracle.expert_mlp(*cache[e], xs[t], 2048, 512)
             acc = (acc + ref_w[t, kk] * c).astype(np.float32)
         ref[t] = acc
+    return ref
+
+
+@pytest.mark.parametrize("max_tokens,tokens", [(1, 1), (3, 3), (4, 2), (32, 32), (37, 37)])
+def test_grouped_forward_model_geometry(oracle, X, max_tokens, tokens):
+    g = X.MoeGeometry.qwen3_6(32, max_tokens)
+    layer = make_layer(oracle, g, seed=500)
+    x = activations(12, max_tokens, 2048, tokens)
+    r = oracle.Xorshift64Star(0xA11 + tokens)
+    logits = np.stack([r.vec_f32(256, -8.0, 8.0) for _ in range(tokens)])
+    out, ids, w, _ = _grouped(X, oracle, g, layer, x, tokens, logits)
+    ref_ids, ref_w = oracle.route_batch(logits, 8)
+    assert np.array_equal(ids, ref_ids.astype(np.int32))
+    ref = _naive_model_ref(oracle, layer.host, x.cpu().numpy(), ref_ids, ref_w, tokens)
     rr = oracle.compare(out[:tokens], ref)
     assert rel_to_peak(out[:tokens], ref) <= DECODE_REL and rr.cosine_similarity >= DECODE_COS, str(rr)
+
+
+@pytest.mark.parametrize("max_tokens,tokens", [(8, 8), (12, 12), (12, 7)])
+def test_exact_decode_regime_matches_naive_forward(oracle, X, max_tokens, tokens):
+    """The exact-decode regime (kernels/moe.rs:5436-5452) pins the flat per-pair kernels at widths that would
+    otherwise take the dispatch tables; the speculative verify windows of 2-12 rows are its callers
+    (tests/moe_differential.rs:1392-1402).  Checked directly against the CPU reference at the fp32 gate."""
+    g = X.MoeGeometry.qwen3_6(32, max_tokens)
+    layer = make_layer(oracle, g, seed=510)
+    x = activations(14, max_tokens, 2048, tokens)
+    r = oracle.Xorshift64Star(0xE8AC7 + tokens)
+    logits = np.stack([r.vec_f32(256, -8.0, 8.0) for _ in range(tokens)])
+    out, ids, w, b = _grouped(X, oracle, g, layer, x, tokens, logits, exact=True)
+    ref_ids, ref_w = oracle.route_batch(logits, 8)
+    assert np.array_equal(ids, ref_ids.astype(np.int32))
+    assert np.abs(w - ref_w).max() <= 1e-6
+    ref = _naive_model_ref(oracle, layer.host, x.cpu().numpy(), ref_ids, ref_w, tokens)
+    rr = oracle.compare(out[:tokens], ref)
+    assert rel_to_peak(out[:tokens], ref) <= DECODE_REL and rr.cosine_similarity >= DECODE_COS, str(rr)
+    assert np.all(out[tokens:] == 0)
+    # the regime really is the flat one: no dispatch table was built for this pass
+    assert int(b.num_tokens_post_pad().cpu().numpy()[0]) == 0
+    # and the same pass without the pin (dispatch-table kernels) gives the same bits
+    out2, ids2, _, _ = _grouped(X, oracle, g, layer, x, tokens, logits, exact=False)
+    assert np.array_equal(ids2, ids) and np.array_equal(out2.view(np.uint32), out.view(np.uint32))
 
 
 def test_all_tokens_to_one_expert_collides_in_one_dispatch_run(oracle, X):

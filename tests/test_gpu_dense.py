@@ -108,3 +108,63 @@ def test_long_row_kernel_equals_the_plain_one(dense, max_tokens, tokens):
         outs.append(out.cpu().numpy().copy())
     assert outs[0][:tokens].any() and not outs[0][tokens:].any()
     assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+
+
+CHAIN_LAYERS = 64
+
+
+@pytest.fixture(scope="module")
+def dense_chain():
+    """configs[4]'s chain: 64 independently seeded layers (14 GB of Q6_K), each block's l_out the next block's input."""
+    import torch
+    import llmxabe_amd as X
+
+    H, I = 5120, 17408
+    q = X.ExpertQuant.Q6K
+    layers = []
+    for l in range(CHAIN_LAYERS):
+        s = 70_000 + 10 * l
+        t = lambda r: X.QuantTensor(X.synth_quant(q, s + r, H * I, 0.02), q)
+        layers.append(X.DenseFfnLayerWeights(1.0 + X.synth_normal_f32(s, H, 0.1), t(1), t(2), t(3)))
+    torch.cuda.synchronize()
+    return X, layers, H, I
+
+
+def _run_chain(X, layers, H, I, x_rows, max_tokens, keep=()):
+    import torch
+
+    blk = X.DenseFfnBlock(H, I, max_tokens)
+    t = x_rows.shape[0]
+    cur = torch.zeros(max_tokens, H, device="cuda")
+    cur[:t] = x_rows
+    ffn = torch.zeros_like(cur)
+    kept = {}
+    for l, w in enumerate(layers):
+        nxt = torch.zeros_like(cur)
+        blk.forward(w, cur, t, ffn, nxt)
+        if l in keep:
+            kept[l] = (cur[:t].cpu().numpy(), nxt[:t].cpu().numpy())
+        cur = nxt
+    torch.cuda.synchronize()
+    return cur[:t].cpu().numpy(), kept
+
+
+def test_dense_chain_is_batch_invariant_end_to_end(oracle, dense_chain):
+    """Decode at batch 8 and batch 1 through all 64 layers: each token alone equals its row in the batch bit
+    for bit at the END of the chain (so at every layer), and sampled layers equal the oracle on the device's
+    own layer input."""
+    X, layers, H, I = dense_chain
+    xs = X.synth_normal_f32(54, 8 * H, 1.0).view(8, H)
+    keep = (0, CHAIN_LAYERS // 2, CHAIN_LAYERS - 1)
+    batch, kept = _run_chain(X, layers, H, I, xs, 8, keep=keep)
+    assert np.all(np.isfinite(batch)) and np.abs(batch).max() > 0
+    for t in range(8):
+        alone, _ = _run_chain(X, layers, H, I, xs[t:t + 1], 1)
+        assert np.array_equal(alone[0].view(np.uint32), batch[t].view(np.uint32)), f"token {t} differs alone vs in the batch"
+    c = lambda t: t.cpu().numpy()
+    for l in keep:
+        w = layers[l]
+        x_in, l_dev = kept[l]
+        _, _, l_ref = oracle.dense_block_forward(H, I, 1e-6, c(w.post_norm), c(w.gate.bytes), c(w.up.bytes),
+                                                 c(w.down.bytes), x_in[:2], threads=16)
+        assert rel_to_peak(l_dev[:2], l_ref) <= DECODE_REL, l

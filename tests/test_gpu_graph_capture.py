@@ -99,3 +99,36 @@ def test_dense_block_and_lm_head_replay(oracle, X):
     torch.cuda.synchronize()
     want = [logits.view(torch.int32).clone(), out.clone()]
     _replays(torch, stream, head_pass, [logits, out], lambda: (logits.fill_(-1.0), out.fill_(-5)), want, "LM head + argmax")
+
+
+def test_token_count_change_inside_a_capture_is_refused(oracle, X):
+    """set_valid_tokens is a host-to-device copy: recorded into a graph it would publish, on every replay, whatever
+    its source held then.  The count is published before the capture (kernels/moe.rs:5473-5491); a forward whose
+    count differs from the published one while the stream is capturing is refused and records nothing, and the
+    same forward outside the capture still works."""
+    import torch
+
+    g = X.MoeGeometry.qwen3_6(32, 4)
+    layer = make_layer(oracle, g, seed=8900)
+    blk = X.MoeBlock(g)
+    x = activations(8901, 4, 2048, 4)
+    ffn, lout = torch.zeros_like(x), torch.zeros_like(x)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        blk.forward(layer.dev, x, 4, ffn, lout)       # publishes 4
+        stream.synchronize()
+        want = lout.clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            with pytest.raises(X.moe.InvalidArgument, match="publish the count before the capture begins"):
+                blk.forward(layer.dev, x, 2, ffn, lout)
+            blk.forward(layer.dev, x, 4, ffn, lout)   # unchanged count: nothing to copy, captured normally
+        lout.fill_(float("nan"))
+        graph.replay()
+        stream.synchronize()
+        assert torch.equal(lout.view(torch.int32), want.view(torch.int32))
+        # outside the capture the refused width is served, and the cache was not poisoned by the refusal
+        lout.zero_()
+        blk.forward(layer.dev, x, 2, ffn, lout)
+        stream.synchronize()
+        assert torch.equal(lout[:2].view(torch.int32), want[:2].view(torch.int32)) and not bool(lout[2:].any())

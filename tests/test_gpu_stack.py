@@ -81,9 +81,11 @@ def test_each_layer_matches_the_oracle_on_the_devices_input(oracle, stack):
         assert rel_to_peak(lout.cpu().numpy(), ref.l_out) <= 2e-5, l
 
 
-def test_prefill_8192_chunk_through_some_layers(oracle, stack):
-    """The 8192-token prefill chunk (B = 64): finite, routed exactly on the device's logits, and a sample of
-    rows of one layer checked against the oracle at the matrix-core tolerance."""
+def test_prefill_8192_chunk_through_the_whole_stack(oracle, stack):
+    """The 8192-token prefill chunk (B = 64) through every layer of the stack, each block's l_out the next
+    block's input: finite everywhere; every layer's dispatch tables hold each live (token, k) exactly once; on
+    sampled layers ALL 8192 rows are routed exactly as the CPU reference routes the device's own logits; and a
+    sample of rows of those layers is checked against the oracle block at the matrix-core tolerance."""
     import torch
 
     X, layers = stack
@@ -93,29 +95,37 @@ def test_prefill_8192_chunk_through_some_layers(oracle, stack):
     blk = X.MoeBlock(g)
     cur = activations(63, T, 2048)
     ffn = torch.zeros_like(cur)
-    for w in layers[:3]:
+    sampled = sorted({0, 2, LAYERS // 2, LAYERS - 1})
+    rows = [0, 63, 64, 4097, 8191]
+    kept = {}
+    all_pairs = np.arange(T * 8)
+    for l, w in enumerate(layers):
         nxt = torch.zeros_like(cur)
-        x_in = cur
         blk.forward(w, cur, T, ffn, nxt)
+        b = blk.buffers()
+        sorted_ids = b.sorted_token_ids().cpu().numpy()
+        n = int(b.num_tokens_post_pad().cpu().numpy()[0])
+        assert n % 64 == 0 and n <= sorted_ids.size, l
+        live = sorted_ids[:n][sorted_ids[:n] != T * 8]
+        assert live.size == T * 8 and np.array_equal(np.sort(live), all_pairs), f"layer {l}: dispatch tables"
+        assert np.all(sorted_ids[n:] == T * 8), f"layer {l}: sentinel fill"
+        if l in sampled:
+            kept[l] = dict(x=cur[rows].cpu().numpy(), out=nxt[rows].cpu().numpy(),
+                           logits=blk.router_logits().view(T, 256).cpu().numpy(),
+                           ids=b.topk_ids().view(T, 8).cpu().numpy())
+        assert bool(torch.isfinite(nxt).all()), f"layer {l}: non-finite l_out"
         cur = nxt
     torch.cuda.synchronize()
-    assert torch.isfinite(cur).all()
-    w = layers[2]
-    rows = [0, 63, 64, 4097, 8191]
-    dev_logits = blk.router_logits().view(T, 256)[rows].cpu().numpy()
-    ids = blk.buffers().topk_ids().view(T, 8)[rows].cpu().numpy()
     c = lambda t: t.cpu().numpy()
-    host = oracle.MoeWeights(
-        num_experts=256, top_k=8, hidden=2048, intermediate=512, eps=1e-6, post_norm=c(w.post_norm), router_f32=None,
-        router_q8=c(w.router), gate_exps=c(w.gate_exps.bytes), up_exps=c(w.up_exps.bytes), down_exps=c(w.down_exps.bytes),
-        shared_gate_inp=c(w.shared_gate_inp), shared_gate=c(w.shared_gate.bytes), shared_up=c(w.shared_up.bytes),
-        shared_down=c(w.shared_down.bytes))
-    ref = oracle.moe_block_forward(host, x_in[rows].cpu().numpy(), logits_override=dev_logits, threads=8)
-    assert np.array_equal(ids, ref.topk_ids.astype(np.int32))
-    assert rel_to_peak(cur[rows].cpu().numpy(), ref.l_out) <= 1e-3
-    # the dispatch tables of that pass: every live (token, k) exactly once
-    b = blk.buffers()
-    sorted_ids = b.sorted_token_ids().cpu().numpy()
-    n = int(b.num_tokens_post_pad().cpu().numpy()[0])
-    live = sorted_ids[:n][sorted_ids[:n] != T * 8]
-    assert live.size == T * 8 and np.array_equal(np.sort(live), np.arange(T * 8))
+    for l, k in kept.items():
+        ref_ids, _ = oracle.route_batch(k["logits"], 8)
+        assert np.array_equal(k["ids"], ref_ids.astype(np.int32)), f"layer {l}: routing differs from route_batch(device logits)"
+        w = layers[l]
+        host = oracle.MoeWeights(
+            num_experts=256, top_k=8, hidden=2048, intermediate=512, eps=1e-6, post_norm=c(w.post_norm), router_f32=None,
+            router_q8=c(w.router), gate_exps=c(w.gate_exps.bytes), up_exps=c(w.up_exps.bytes),
+            down_exps=c(w.down_exps.bytes), shared_gate_inp=c(w.shared_gate_inp), shared_gate=c(w.shared_gate.bytes),
+            shared_up=c(w.shared_up.bytes), shared_down=c(w.shared_down.bytes))
+        ref = oracle.moe_block_forward(host, k["x"], logits_override=k["logits"][rows], threads=8)
+        assert np.array_equal(k["ids"][rows], ref.topk_ids.astype(np.int32)), l
+        assert rel_to_peak(k["out"], ref.l_out) <= 1e-3, l

@@ -159,6 +159,37 @@ def test_q6k_quantizer_formula_independently(oracle):
         assert np.array_equal(np_dequant_q6k(one).astype(np.int32), codes)
 
 
+def test_quantizers_round_exact_halves_away_from_zero(oracle):
+    """`f32::round` is half-away-from-zero (quant.rs:75-88, :495-567); C's rintf / numpy's round go to even.
+    Inputs built so that the quotient is exactly k + 0.5 in fp32, where the two rules differ; the expected
+    codes are written out by hand."""
+    # Q8_0: amax 127 -> d = 1, 1/d = 1, so v * inv_d == v
+    x = np.zeros(32, np.float32)
+    x[:12] = [127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5, -3.5, 126.5, -126.5, 4.5]
+    b = oracle.quantize_row(oracle.Q8_0, x)
+    assert b[:2].view(np.float16)[0] == np.float16(1.0)
+    assert b[2:14].view(np.int8).tolist() == [127, 1, 2, 3, -1, -2, -3, 4, -4, 127, -127, 5]
+    assert np.rint(x[1:9]).tolist() == [0, 2, 2, -0, -2, -2, 4, -4]          # what half-to-even would have stored
+    # Q6_K: amax 4064 -> d = 4064 / (32 * 127) = 1.  Group 0 (positions 0..15): amax 4064 -> sc = 127, and
+    # x = 127 * (k + 0.5) gives the quotient k + 0.5 exactly.  Group 1 (positions 16..31): amax 336 = 32 * 10.5,
+    # so the SCALE itself sits on a half: 11 away from zero, 10 to even; its codes then divide by 11.
+    x = np.zeros(256, np.float32)
+    x[0] = 4064.0
+    x[1:7] = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5], np.float32) * np.float32(127.0)
+    x[16] = 336.0
+    x[17:21] = np.array([0.5, 1.5, -0.5, -2.5], np.float32) * np.float32(11.0)
+    blk = oracle.quantize_row(oracle.Q6K, x)
+    assert blk[208:210].view(np.float16)[0] == np.float16(1.0)
+    scales = blk[192:208].view(np.int8)
+    assert scales[0] == 127 and scales[1] == 11 and not scales[2:].any()
+    one = blk.copy()
+    one[192:208] = 1                                                          # read the raw codes back out
+    codes = np_dequant_q6k(one).astype(np.int32)
+    assert codes[:7].tolist() == [31, 1, 2, 3, -1, -2, -3]                    # 4064/127 = 32 clamps to 31
+    assert codes[16:21].tolist() == [31, 1, 2, -1, -3]                        # 336/11 = 30.55 -> 31
+    assert not codes[7:16].any() and not codes[21:].any()
+
+
 def test_q6k_bytes_round_trip(oracle):
     # quant.rs:1319-1337
     x = ((np.arange(256) % 61).astype(np.float32) - 30.0) * np.float32(0.1)
