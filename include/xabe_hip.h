@@ -264,6 +264,20 @@ int xabe_moe_block_forward_stage(xabe_moe_block* blk, void* stream, const xabe_m
                                  const float* residual, size_t residual_len, const float* logit_bias, float* ffn_out,
                                  size_t ffn_out_len, float* l_out, size_t l_out_len, int stage);
 int xabe_moe_block_tensor_cores_enabled(const xabe_moe_block* blk);      /* B:1008-1010 */
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code that builds its launches
+ * under hipGraph capture without handles, tight serving loops, harnesses that forbid hipMalloc): xabe_moe_block_forward
+ * at decode widths with the block's working set (normalised rows, logits, selections, intermediates, the live-token
+ * count) in a device array the library holds statically (1.4 MB per GPU, until the process ends) instead of in buffers
+ * that xabe_moe_block_new allocates.  No handle, no hipMalloc/hipFree, the same three launches and the same bits.
+ * Serves max_tokens <= 32, hidden <= 2048, intermediate <= 512, <= 512 experts, top-k <= 8, in the shapes and
+ * formats of the three-launch decode block; anything larger is XABE_ERR_UNSUPPORTED_GEOMETRY.  The live-token count
+ * is published by a one-thread kernel, so the call may be captured.  All calls on one GPU share that GPU's array:
+ * calls that overlap on one GPU race.  The first call on a device resolves the array's address there; make it
+ * outside a capture. */
+int xabe_moe_block_forward_noalloc(const xabe_moe_geometry* geometry, float eps, void* stream,
+                                   const xabe_moe_layer_weights* w, const float* residual, size_t residual_len,
+                                   size_t tokens, const float* logit_bias, float* ffn_out, size_t ffn_out_len, float* l_out,
+                                   size_t l_out_len);
 /* Read-back accessors (B:1023-1060): device pointer + element count. */
 const float* xabe_moe_block_normed(const xabe_moe_block* blk, size_t* len);
 const float* xabe_moe_block_router_logits(const xabe_moe_block* blk, size_t* len);

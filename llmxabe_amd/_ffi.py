@@ -115,6 +115,8 @@ _SIGNATURES = {
     "xabe_moe_block_free": (None, [vp]),
     "xabe_moe_block_publish_tokens": (C.c_int, [vp, vp, sz]),
     "xabe_moe_block_forward": (C.c_int, [vp, vp, C.POINTER(MoeLayerWeightsC), vp, sz, sz, vp, vp, sz, vp, sz]),
+    "xabe_moe_block_forward_noalloc": (C.c_int, [C.POINTER(Geometry), C.c_float, vp, C.POINTER(MoeLayerWeightsC), vp, sz, sz, vp, vp, sz,
+                                                 vp, sz]),
     "xabe_moe_block_disable_tensor_cores": (C.c_int, [vp]),
     "xabe_moe_block_set_exact_decode_regime": (C.c_int, [vp, C.c_int]),
     "xabe_moe_block_set_fused_decode": (C.c_int, [vp, C.c_int]),

@@ -95,6 +95,16 @@ class MoeBlock:
         return MoeBuffers(_ffi.lib().xabe_moe_block_buffers(self._h), owner=False)
 
 
+def moe_block_forward_noalloc(geometry: MoeGeometry, w: MoeLayerWeights, residual, tokens: int, ffn_out, l_out,
+                              logit_bias=None, eps: float = DEFAULT_RMS_EPS):
+    """`MoeBlock.forward` at decode widths without a block: the working set lives in a device array the library
+    holds statically, so the call allocates nothing (no counterpart in the reference; see the header)."""
+    cw = w._c()
+    check(_ffi.lib().xabe_moe_block_forward_noalloc(C.byref(geometry._c()), eps, _stream(), C.byref(cw), _ptr(residual),
+                                                    residual.numel(), tokens, _ptr(logit_bias), _ptr(ffn_out),
+                                                    ffn_out.numel(), _ptr(l_out), l_out.numel()))
+
+
 @dataclass
 class DenseFfnLayerWeights:
     post_norm: torch.Tensor

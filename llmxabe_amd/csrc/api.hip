@@ -282,6 +282,22 @@ static int launch_expert(const xabe_moe_kernels* k, Mode mode, int quant, int nm
   return XABE_OK;
 }
 
+// the reference's checks on a geometry, in its order, with its reasons (kernels/moe.rs:5043-5111)
+int validate_geometry(const xabe_moe_geometry& g) {
+  if (g.block_size == 0) return bad_geometry(g, "block_size must be non-zero");
+  if (g.experts_per_token == 0) return bad_geometry(g, "experts_per_token must be non-zero");
+  if (g.experts_per_token > g.num_experts) return bad_geometry(g, "experts_per_token must not exceed num_experts");
+  if (g.max_tokens == 0) return bad_geometry(g, "max_tokens must be non-zero");
+  if (g.hidden == 0 || g.intermediate == 0) return bad_geometry(g, "hidden and intermediate must be non-zero");
+  if (g.hidden % 128 != 0) return bad_geometry(g, "hidden must be a multiple of the 128-element tile");
+  if (g.intermediate % 128 != 0) return bad_geometry(g, "intermediate must be a multiple of the 128-element tile");
+  if (g.block_size > 64) return bad_geometry(g, "block_size exceeds the slots the tensor-core tile stages");
+  if (xabe_moe_geometry_expert_block_capacity(&g) > 65535)
+    return bad_geometry(g, "dispatch-block capacity exceeds the 65535 grid.y limit");
+  if (g.max_tokens > 65535) return bad_geometry(g, "max_tokens exceeds the 65535 grid limit");
+  return XABE_OK;
+}
+
 }  // namespace xabe
 
 using namespace xabe;
@@ -386,18 +402,7 @@ int xabe_to_device_layout(int quant, const uint8_t* bytes, size_t len, uint8_t* 
 int xabe_moe_kernels_new(const xabe_moe_geometry* geometry, xabe_moe_kernels** out) {
   if (!geometry || !out) return set_error(XABE_ERR_INVALID_ARGUMENT, "MoeKernels::new: null pointer");
   const xabe_moe_geometry g = *geometry;
-  // the reference's checks, in its order, with its reasons (kernels/moe.rs:5043-5111)
-  if (g.block_size == 0) return bad_geometry(g, "block_size must be non-zero");
-  if (g.experts_per_token == 0) return bad_geometry(g, "experts_per_token must be non-zero");
-  if (g.experts_per_token > g.num_experts) return bad_geometry(g, "experts_per_token must not exceed num_experts");
-  if (g.max_tokens == 0) return bad_geometry(g, "max_tokens must be non-zero");
-  if (g.hidden == 0 || g.intermediate == 0) return bad_geometry(g, "hidden and intermediate must be non-zero");
-  if (g.hidden % 128 != 0) return bad_geometry(g, "hidden must be a multiple of the 128-element tile");
-  if (g.intermediate % 128 != 0) return bad_geometry(g, "intermediate must be a multiple of the 128-element tile");
-  if (g.block_size > 64) return bad_geometry(g, "block_size exceeds the slots the tensor-core tile stages");
-  if (xabe_moe_geometry_expert_block_capacity(&g) > 65535)
-    return bad_geometry(g, "dispatch-block capacity exceeds the 65535 grid.y limit");
-  if (g.max_tokens > 65535) return bad_geometry(g, "max_tokens exceeds the 65535 grid limit");
+  XABE_TRY(validate_geometry(g));
 
   int dev = 0;
   XABE_HIP_TRY(hipGetDevice(&dev));

@@ -25,6 +25,7 @@ constexpr size_t kRouteMaxExperts = 512;  // the routing wavefront holds 8 exper
 int set_error(int status, const char* fmt, ...);
 int hip_error(hipError_t e, const char* what);
 std::string geometry_debug(const xabe_moe_geometry& g);
+int validate_geometry(const xabe_moe_geometry& g);  // MoeKernels::new's checks (api.hip)
 
 #define XABE_HIP_TRY(expr)                                  \
   do {                                                      \

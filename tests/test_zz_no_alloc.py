@@ -1,0 +1,78 @@
+"""xabe_moe_block_forward_noalloc (no counterpart in the reference: for callers that cannot allocate device
+memory) against xabe_moe_block_forward, through the C ABI: same bits, on two calls in a row, the second with a
+smaller input; and the size limit is an error, not a fault."""
+import pytest
+
+from util import activations, make_layer, run_block
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(X, oracle, max_tokens, tokens, seed, bias=False):
+    import torch
+
+    g = X.MoeGeometry.qwen3_6(32, max_tokens)
+    layer = make_layer(oracle, g, seed=seed)
+    x = activations(seed + 1, max_tokens, 2048, tokens)
+    lb = X.synth_normal_f32(seed + 2, 256, 1.0) if bias else None
+    want_ffn, want_l = run_block(X.MoeBlock(g), layer, x, tokens, logit_bias=lb)
+    # poisoned outputs: rows past the live tokens must stay untouched, live rows must be overwritten
+    ffn = torch.full_like(x, float("nan"))
+    lout = torch.full_like(x, float("nan"))
+    X.moe_block_forward_noalloc(g, layer.dev, x, tokens, ffn, lout, logit_bias=lb)
+    torch.cuda.synchronize()
+    assert want_l[:tokens].abs().max() > 0
+    assert torch.equal(ffn[:tokens].view(torch.int32), want_ffn[:tokens].view(torch.int32)), (max_tokens, tokens)
+    assert torch.equal(lout[:tokens].view(torch.int32), want_l[:tokens].view(torch.int32)), (max_tokens, tokens)
+    assert bool(torch.isnan(ffn[tokens:]).all()) and bool(torch.isnan(lout[tokens:]).all())
+
+
+def test_noalloc_block_equals_the_allocating_block_on_consecutive_calls(oracle):
+    import llmxabe_amd as X
+
+    _both(X, oracle, 32, 32, 9500)             # the largest pass the scratch array serves
+    _both(X, oracle, 3, 3, 9510, bias=True)    # then a smaller one over the same array (stale contents around it)
+    _both(X, oracle, 8, 5, 9520)               # fewer live tokens than the pass holds
+    _both(X, oracle, 32, 1, 9530)
+
+
+def test_noalloc_block_inside_a_graph(oracle):
+    import torch
+    import llmxabe_amd as X
+
+    g = X.MoeGeometry.qwen3_6(32, 4)
+    layer = make_layer(oracle, g, seed=9540)
+    x = activations(9541, 4, 2048, 3)
+    want_ffn, want_l = run_block(X.MoeBlock(g), layer, x, 3)
+    ffn, lout = torch.zeros_like(x), torch.zeros_like(x)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        X.moe_block_forward_noalloc(g, layer.dev, x, 3, ffn, lout)      # first call on the device: outside the capture
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            X.moe_block_forward_noalloc(g, layer.dev, x, 3, ffn, lout)
+        for rep in range(3):
+            lout.fill_(float("nan"))
+            X.moe_block_forward_noalloc(g, layer.dev, x, 1, ffn, torch.zeros_like(x))   # eager work in between: count 1
+            stream.synchronize()
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(lout[:3].view(torch.int32), want_l[:3].view(torch.int32)), rep
+
+
+def test_noalloc_block_rejects_what_its_array_cannot_hold(oracle):
+    import torch
+    import llmxabe_amd as X
+
+    g = X.MoeGeometry.qwen3_6(32, 4)
+    layer = make_layer(oracle, g, seed=9550)
+    big = X.MoeGeometry.qwen3_6(32, 33)
+    x = torch.zeros(33, 2048, device="cuda")
+    with pytest.raises(X.moe.UnsupportedGeometry, match="serves at most 32 tokens"):
+        X.moe_block_forward_noalloc(big, layer.dev, x, 33, torch.zeros_like(x), torch.zeros_like(x))
+    x4 = torch.zeros(4, 2048, device="cuda")
+    with pytest.raises(X.moe.TooManyTokens):
+        X.moe_block_forward_noalloc(g, layer.dev, x4, 5, torch.zeros_like(x4), torch.zeros_like(x4))
+    with pytest.raises(X.moe.BufferLength):
+        X.moe_block_forward_noalloc(g, layer.dev, x4[:3], 3, torch.zeros_like(x4), torch.zeros_like(x4))
