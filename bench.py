@@ -29,6 +29,79 @@ SHARED_BYTES = 3 * (512 * 2048 // 32 * 34)      # shared expert, Q8_0
 ROUTER_BYTES = 256 * 2048 // 32 * 34            # router, Q8_0
 
 
+MIN_TIMED_STEPS = 320   # the headline's timed region never covers fewer block passes than this (~11 ms)
+
+
+def routing_margin(logits):
+    """min over tokens of p(8th selected) - p(9th): how close the top-8 / top-9 decision of `route_token`
+    (crates/xabe-kernels/src/moe/router.rs:32-76) comes to a tie on these logits; float64 softmax on the host."""
+    import numpy as np
+
+    l = np.asarray(logits, np.float64)
+    e = np.exp(l - l.max(axis=1, keepdims=True))
+    p = np.sort(e / e.sum(axis=1, keepdims=True), axis=1)[:, ::-1]
+    ls = np.sort(l, axis=1)[:, ::-1]
+    return float((p[:, 7] - p[:, 8]).min()), float((ls[:, 7] - ls[:, 8]).min())
+
+
+def source_digest():
+    """Digest of the kernel sources the counter-derived `traffic` figure was taken on: a figure from another
+    version of the kernels is reported as stale, not as measured."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in ("decode_block.hip", "decode_kernels.h", "device_common.h", "route_device.h"):
+        with open(os.path.join(ROOT, "llmxabe_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def prefill_leg(X, layers, T, reps, bias=None):
+    """One prefill configuration of the block (eager launches, HIP events on the launch stream, layers rotated)."""
+    import numpy as np
+    import torch
+
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
+    blk = X.MoeBlock(g)
+    blk.publish_tokens(T)
+    x = X.synth_normal_f32(99, T * 2048, 1.0).view(T, 2048)
+    ffn_out, l_out = torch.zeros_like(x), torch.zeros_like(x)
+    extra = {"logit_bias": bias} if bias is not None else {}
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    L = len(layers)
+    with torch.cuda.stream(stream):
+        for i in range(2 * L):
+            blk.forward(layers[i % L], x, T, ffn_out, l_out, **extra)
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            for i in range(L):
+                blk.forward(layers[i], x, T, ffn_out, l_out, **extra)
+        e1.record(stream)
+        e1.synchronize()
+    ms = e0.elapsed_time(e1) / (reps * L)
+    ids = blk.buffers().topk_ids().cpu().numpy().reshape(T, 8)
+    distinct = len(np.unique(ids))
+    byts = distinct * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES + 16384 + T * 2048 * 4 * 3
+    flops = T * 57671680
+    gbps, tflops = byts / (ms * 1e-3) / 1e9, flops / (ms * 1e-3) / 1e12
+    margin_p, margin_l = routing_margin(blk.router_logits().view(T, 256).cpu().numpy())
+    counts = np.bincount(ids.ravel(), minlength=256)
+    out = {"tokens": T, "block_size": g.block_size, "ms_per_block": ms, "tokens_per_s": T / (ms * 1e-3), "steps": reps * L,
+           "layers_rotated": L, "tflops": tflops, "frac_of_mfma_peak": tflops / MFMA_PEAK_TFLOPS, "gbps": gbps,
+           "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS, "bound": "mfma" if T >= 4096 else "hbm",
+           "distinct_experts": distinct, "algorithmic_bytes_per_block": byts, "flops_per_block": flops,
+           "expert_load": {"max": int(counts.max()), "experts_with_at_most_2_tokens": int((counts <= 2).sum())},
+           "routing_margin_min": margin_p, "routing_logit_gap_min": margin_l,
+           "dtype": "f16 operands, f32 accumulate (router f32)", "launch": "eager",
+           "router_bias": "zipf s=1.1 (b_e = -1.1 ln rank_e), seed 5" if bias is not None else None}
+    del blk, x, ffn_out, l_out
+    torch.cuda.empty_cache()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -41,10 +114,13 @@ def main() -> int:
                     help="before the timed region, copy a 256 MiB device buffer this many times: a kernel of known "
                          "traffic against which hardware byte counters of the same run are scaled")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the two prefill legs of the headline run")
+    ap.add_argument("--no-calibration", action="store_true", help="skip the read / matrix-instruction calibration legs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--workload", default="decode_b3", choices=["decode_b3"] + sorted(OTHER_WORKLOADS),
-                    help="decode_b3 is the headline (everything above applies to it); the others are BASELINE's "
-                         "remaining configurations, timed whole-block with HIP events, for profiles and comparison")
+                    help="decode_b3 is the headline: the batch-3 decode block (value, roofline), followed by the "
+                         "8192-token and the skewed 512-token prefill blocks (the `prefill` object); the others are "
+                         "BASELINE's remaining configurations one at a time, for profiles and comparison")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -81,7 +157,10 @@ def main() -> int:
     def one_pass(i):
         blk.forward(layers[i % L], x, T, ffn_out, l_out)
 
-    # ---- timed region: K steps, W warmup ----
+    # ---- timed region: W warmup steps, then K steps (never fewer than MIN_TIMED_STEPS: at 30 us a step, the 20
+    # steps a short run asks for are two graph replays, one scheduler hiccup away from noise); whole replays of the
+    # L-pass graph, so both counts are rounded up to multiples of L.  HIP events on the launch stream give the
+    # figure; the host clock around the same region is reported beside it ----
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for i in range(L):
@@ -94,39 +173,44 @@ def main() -> int:
                 for i in range(L):
                     one_pass(i)
         reps_w = max(1, (args.warmup + L - 1) // L)
-        reps = max(1, (args.steps + L - 1) // L)
+        reps = max(1, (max(args.steps, MIN_TIMED_STEPS) + L - 1) // L)
         steps = reps * L
         for _ in range(reps_w):
             graph.replay() if graph else [one_pass(i) for i in range(L)]
         stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        e0.record(stream)
         for _ in range(reps):
             graph.replay() if graph else [one_pass(i) for i in range(L)]
-        stream.synchronize()
-        dt = time.perf_counter() - t0
+        e1.record(stream)
+        e1.synchronize()
+        wall = time.perf_counter() - t0
+        dt = e0.elapsed_time(e1) * 1e-3
     ms_per_step = dt / steps * 1e3
     tokens_per_s = T * steps / dt
 
-    # ---- algorithmic bytes of one step (distinct experts from topk_ids of each layer) ----
-    distinct = []
+    # ---- algorithmic bytes of one step (distinct experts from topk_ids of each layer), and how close the routing
+    # decision of each pass came to a tie ----
+    distinct, margins, gaps = [], [], []
     with torch.cuda.stream(stream):
         for i in range(L):
             one_pass(i)
             stream.synchronize()
             ids = blk.buffers().topk_ids().cpu().numpy().reshape(T, 8)
             distinct.append(len(np.unique(ids)))
+            mp, ml = routing_margin(blk.router_logits().view(T, 256).cpu().numpy())
+            margins.append(mp)
+            gaps.append(ml)
     d_active = float(np.mean(distinct))
     step_bytes = d_active * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES + 16384 + T * 2048 * 4 * 3
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     # ---- the three launches of the block, each timed alone (HIP events on the launch stream, graph replay
     # over the same rotated layers); the dominant one is launch 1: route + routed gate/up, which streams
-    # two of the three matrices of every (token, k) pair ----
-    pairs = T * 8
-    chunks = (T + 1) // 2  # launch 0 reads the router and the shared gate/up once per chunk of two tokens
-    stage_bytes = [chunks * (ROUTER_BYTES + 2 * (SHARED_BYTES // 3)),
-                   pairs * 2 * EXPERT_MATRIX_BYTES,
-                   pairs * EXPERT_MATRIX_BYTES + T * (SHARED_BYTES // 3)]
+    # two of the three matrices of every distinct expert selected (and the shared expert's gate/up pair) ----
+    chunks = (T + 1) // 2  # token chunks of two share one pass over the router and shared gate/up
+    stage_bytes = decode_stage_bytes(T, d_active, chunks)
     stage_us = []
     with torch.cuda.stream(stream):
         one_pass(0)  # leaves layer 0's logits, normalised rows and shared activations for stages 1 and 2
@@ -153,15 +237,22 @@ def main() -> int:
             stage_us.append(e0.elapsed_time(e1) * 1e3 / (kreps * L))
     kern_bytes, kern_us = stage_bytes[1], stage_us[1]
     achieved = kern_bytes / (kern_us * 1e-6) / 1e9
-    traffic = None
+    # HBM bytes per launch of the dominant kernel from hardware counters: taken in separate `rocprofv3 --pmc` runs of
+    # this command (profiles/moe_block_decode_b3_hbm_traffic.md), valid only for the kernel sources it was taken on
+    traffic, traffic_note = None, "no counter profile for this workload"
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
+    if os.path.exists(tpath) and T == 3:
         try:
-            traffic = json.load(open(tpath)).get("k_decode_up_b3_bytes_per_launch")
-        except Exception:
-            traffic = None
-    stage_names = ["k_decode_logits (router logits + shared gate/up)", "k_decode_up (route + routed gate/up)",
-                   "k_decode_down (routed + shared down, combine)"]
+            tj = json.load(open(tpath))
+            if tj.get("kernel_source_digest") == source_digest():
+                traffic = tj.get("k_decode_up_b3_bytes_per_launch")
+                traffic_note = "rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE per dispatch, scaled by a 256 MiB copy (profiles/moe_block_decode_b3_hbm_traffic.md)"
+            else:
+                traffic_note = "stale: profiles/traffic.json was taken on other kernel sources (digest %s, now %s)" % (
+                    tj.get("kernel_source_digest"), source_digest())
+        except Exception as e:  # noqa: BLE001
+            traffic_note = f"unreadable profiles/traffic.json: {e}"
+    stage_names = DECODE_STAGE_NAMES
 
     out = {
         "metric": "MoE-block tokens/s at 1 GPU; decode HBM GB/s %peak; prefill MFMA util %",
@@ -179,20 +270,63 @@ def main() -> int:
         "config": {"workload": "moe_block_decode_b3" if T == 3 else f"moe_block_decode_b{T}", "tokens": T,
                    "num_experts": 256, "top_k": 8, "hidden": 2048, "intermediate": 512, "expert_quant": "Q6_K",
                    "shared_and_router_quant": "Q8_0", "layers_rotated": L, "launch": "eager" if args.no_graph else "hipGraph"},
+        "timing": {"steps_requested": args.steps, "warmup_requested": args.warmup, "steps_timed": steps,
+                   "warmup_run": reps_w * L, "min_timed_steps": MIN_TIMED_STEPS,
+                   "method": f"HIP events on the launch stream around {reps} replays of a {L}-pass hipGraph "
+                             f"(whole replays: both counts are rounded up to multiples of {L}; the timed region is never "
+                             f"shorter than {MIN_TIMED_STEPS} steps)",
+                   "timed_region_ms": dt * 1e3, "host_clock_ms_per_step": wall / steps * 1e3},
         "decode": {"distinct_experts_per_step": d_active, "algorithmic_bytes_per_step": step_bytes,
                    "block_gbps": step_gbps, "block_frac_of_hbm_peak": step_gbps / HBM_PEAK_GBPS,
                    "roofline_tokens_per_s": T / (step_bytes / (HBM_PEAK_GBPS * 1e9)),
-                   "frac_of_roofline": tokens_per_s / (T / (step_bytes / (HBM_PEAK_GBPS * 1e9)))},
-        "roofline": {"kernel": "k_decode_up<Q6_K,hidden 2048> (route + routed gate/up)", "bound": "hbm", "achieved": achieved,
+                   "frac_of_roofline": tokens_per_s / (T / (step_bytes / (HBM_PEAK_GBPS * 1e9))),
+                   "routing_margin_min": float(np.min(margins)), "routing_logit_gap_min": float(np.min(gaps))},
+        "roofline": {"kernel": DECODE_DOMINANT_KERNEL, "bound": "hbm", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
+                     "traffic_source": traffic_note,
                      "algorithmic_bytes_per_launch": kern_bytes, "launch_us": kern_us},
         "launches": [{"kernel": n, "launch_us": u, "algorithmic_bytes": int(bts), "gbps": bts / (u * 1e-6) / 1e9}
                      for n, u, bts in zip(stage_names, stage_us, stage_bytes)],
     }
+    del graph, blk
 
-    # ---- what this box can do, next to the nominal peaks: a pure coalesced 16-byte-per-lane read of 2 GiB
-    # (eight times the 256 MB Infinity Cache) and a register-resident fp16 matrix-instruction loop, both
-    # kernels of this library's calibrate.hip; and, for comparison, two library routines
+    # ---- the prefill half of the metric: the 8192-token chunk (MFMA-bound) and configs[2]'s 512-token chunk under a
+    # seeded Zipf(1.1) router bias (HBM-bound), on the first layers of the same weight sets ----
+    if not args.no_prefill:
+        rank = np.random.default_rng(5).permutation(256) + 1
+        zipf = torch.from_numpy((-1.1 * np.log(rank)).astype(np.float32)).cuda()
+        out["prefill"] = {"tokens_8192": prefill_leg(X, layers[:2], 8192, 20),
+                          "tokens_512_zipf": prefill_leg(X, layers[:4], 512, 40, bias=zipf)}
+        out["prefill"]["mfma_util_pct"] = 100.0 * out["prefill"]["tokens_8192"]["frac_of_mfma_peak"]
+
+    if not args.no_calibration:
+        out["calibration"] = calibration(X, stream)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(layers[0], g, x, T, args.cpu_seconds)
+    print(json.dumps(out))
+    return 0
+
+
+DECODE_STAGE_NAMES = ["k_decode_logits (router logits + shared gate/up)", "k_decode_up (route + routed gate/up)",
+                      "k_decode_down (routed + shared down, combine)"]
+DECODE_DOMINANT_KERNEL = "k_decode_up<Q6_K,hidden 2048> (route + routed gate/up)"
+
+
+def decode_stage_bytes(T, d_active, chunks):
+    """Algorithmic bytes of the three decode launches: every distinct selected expert's matrices once, the router and
+    the shared expert's matrices once per launch that reads them (re-reads by further token chunks come out of cache
+    and are not algorithmic)."""
+    return [ROUTER_BYTES + 2 * (SHARED_BYTES // 3),
+            d_active * 2 * EXPERT_MATRIX_BYTES,
+            d_active * EXPERT_MATRIX_BYTES + SHARED_BYTES // 3]
+
+
+def calibration(X, stream):
+    """What this box can do, next to the nominal peaks: a pure coalesced 16-byte-per-lane read of 2 GiB (eight times
+    the 256 MB Infinity Cache) and a register-resident fp16 matrix-instruction loop, both kernels of this library's
+    calibrate.hip; and, for comparison, two library routines."""
+    import torch
+
     with torch.cuda.stream(stream):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         big = torch.ones(1 << 29, dtype=torch.int32, device="cuda")   # 2 GiB
@@ -231,15 +365,10 @@ def main() -> int:
         e1.synchronize()
         gemm_tflops = 5 * 2 * 8192 ** 3 / (e0.elapsed_time(e1) * 1e-3) / 1e12
         del ma, mb
-    out["calibration"] = {"hbm_read_gbps": read_gbps, "hbm_read_what": "coalesced 16-byte-per-lane read of 2 GiB (xabe_calibrate_hbm_read)",
-                          "mfma_f16_tflops": mfma_tflops, "mfma_f16_what": "register-resident v_mfma_f32_32x32x16_f16 loop, two wavefronts per SIMD (xabe_calibrate_mfma_f16)",
-                          "device_copy_gbps": copy_gbps, "device_copy_what": "torch copy of 1 GiB, bytes read + written",
-                          "fp16_gemm_tflops": gemm_tflops, "fp16_gemm_what": "torch.matmul 8192^3 fp16 (hipBLASLt)"}
-
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(layers[0], g, x, T, args.cpu_seconds)
-    print(json.dumps(out))
-    return 0
+    return {"hbm_read_gbps": read_gbps, "hbm_read_what": "coalesced 16-byte-per-lane read of 2 GiB (xabe_calibrate_hbm_read)",
+            "mfma_f16_tflops": mfma_tflops, "mfma_f16_what": "register-resident v_mfma_f32_32x32x16_f16 loop, two wavefronts per SIMD (xabe_calibrate_mfma_f16)",
+            "device_copy_gbps": copy_gbps, "device_copy_what": "torch copy of 1 GiB, bytes read + written",
+            "fp16_gemm_tflops": gemm_tflops, "fp16_gemm_what": "torch.matmul 8192^3 fp16 (hipBLASLt)"}
 
 
 MFMA_PEAK_TFLOPS = 2500.0
