@@ -44,6 +44,11 @@ constexpr int kMaxInter = 512;    // intermediate width staged in LDS by k_decod
 // of weights of one step, so more steps against the same registers cut what the launch pulls out of L2, at the
 // price of fewer workgroups.  Measured per width (launch A, us, depth 1 / 2 / 4): one token 5.2 / 5.3 / 6.6, three
 // 7.7 / 6.5 / 8.4, eight 14.2 / 9.4 / 8.4, sixteen - / 15.7 / 11.7.
+// Row steps per workgroup of the third launch (two wavefronts each): two, i.e. eight rows of the 2048-wide block.
+// Four (half as many workgroups, each staging the token's nine activation rows for twice as many rows) measured
+// slower or equal at every width: one token 22.3 against 20.9 us per block, three 32.6 / 31.2, eight 63.8 / 61.8,
+// thirty-two 195.7 / 185.6.
+constexpr int kDownSteps = 2;
 static int logits_depth(int max_tokens) { return max_tokens <= 1 ? 1 : max_tokens <= 6 ? 2 : 4; }
 
 #ifdef XABE_TRACE_ITEMS
@@ -84,59 +89,91 @@ struct DecodeArgs {
   int tiles_r, tiles_s, tiles_g, tiles_d;  // row tiles: router, shared gate/up (launch A), gate/up (B), down (C)
 };
 
-// One step (RPS rows of K = 2048 / RPS elements) of a matrix, or of a gate/up pair, against TC tokens whose
-// rows are normalised on load.  Issues every load before the first use.
+// Row tiles of the first launch: D steps (RPS rows of K = 2048 / RPS elements each) per wavefront of a matrix, or of
+// a gate/up pair, against the TC tokens of the workgroup's chunk, whose rows are normalised on the way in.
 //   NM = 2: out[t][row] = silu(gate . x_t) * (up . x_t);   NM = 1: out[t][row] = (w . x_t) (+ bias[row]).
-template <int QUANT, int RPS, int TC, int NM, int D = 1>
-__device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, int K,
+// The workgroup's four wavefronts need the same TC rows and the norm weight.  They are fetched once per workgroup, as
+// consecutive 16-byte pieces, and handed to the wavefronts through LDS; each wavefront then derives the RMS scales in
+// the canonical order and normalises its own elements, (x * inv) * w: the stand-alone RMSNorm kernel's values.
+// (Each wavefront fetching its own copy from global memory cost 1.9 us of the launch at three tokens: a lane's 32
+// elements are one cache line, so every one of its eight loads touched 64 lines, and all workgroups of the launch aim
+// at the same few rows.)
+// LDS rows are padded by four floats per 32, so that lanes reading 16-byte pieces 128 bytes apart take different banks.
+constexpr int kXnPad = kStepElems + kStepElems / 8;  // floats per staged row
+__device__ __forceinline__ int xn_at(int e) { return e + 4 * (e >> 5); }
+
+template <int QUANT, int RPS, int TC, int NM, int D>
+__device__ __forceinline__ void tile_normed(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, int K,
                                             int n_rows, int row0, const float* const (&xrow)[TC],
                                             const float* __restrict__ norm_w, float eps, float* const (&out)[TC],
                                             const float* __restrict__ bias, const int* __restrict__ valid_tokens,
-                                            int token0) {
+                                            int token0, float* s_xn) {
   using F = Fmt<QUANT>;
   using Raw = typename F::Raw;
   constexpr int G = 64 / RPS;
-  if (row0 >= n_rows) return;
   const LaneGeom g = lane_geom<QUANT>();
   const int koff = lane_koff<QUANT, RPS>(g, 0);
   const size_t row_bytes = (size_t)(K / F::kBlockElems) * F::kBlockBytes;
-  // Q8_0 / fp32 steps give lane L the elements 32L..32L+31 of the row, which is what the RMS fold takes
-  // from it; Q6_K interleaves a superblock over eight lanes, so the fold needs its own copy.
-  constexpr bool kOwnRms = QUANT == kQ6K;
-  RmsRaw q[kOwnRms ? TC : 1];
-  float x[TC][32], xs[TC][4], nw[32];
-  if constexpr (kOwnRms) {
-#pragma unroll
-    for (int t = 0; t < TC; ++t) rms_load(xrow[t], 0, K, q[t]);
-  }
-#pragma unroll
-  for (int t = 0; t < TC; ++t) lane_x_load<QUANT>(xrow[t], koff, g, x[t]);
-  lane_x_load<QUANT>(norm_w, koff, g, nw);
-  // D steps (RPS rows each) against the same activation registers: the rows' weights are all requested here
+  // the rows' weights first: D steps against the same activation registers, all requested here
+  // (a step past the matrix re-reads its last one and is never stored)
   Raw r[D][NM];
 #pragma unroll
   for (int d = 0; d < D; ++d) {
-    const int rd = min(row0 + d * RPS, n_rows - RPS);  // (a step past the matrix re-reads its last one: never stored)
+    const int rd = min(row0 + d * RPS, n_rows - RPS);
     load_raw<QUANT, true>(w0 + (size_t)rd * row_bytes, true, g, r[d][0]);
     if constexpr (NM == 2) load_raw<QUANT, true>(w1 + (size_t)rd * row_bytes, true, g, r[d][NM - 1]);
   }
+  // the chunk's rows and the norm weight, 16 bytes per thread and piece (K <= 2048: two pieces per thread), as they are
+  const int n4 = K / 4;
+  float* s_nw = s_xn + TC * kXnPad;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int i = (int)threadIdx.x + 256 * j, ic = min(i, n4 - 1);
+    const float4 nq = reinterpret_cast<const float4*>(norm_w)[ic];
+    float4 xq[TC];
+#pragma unroll
+    for (int t = 0; t < TC; ++t) xq[t] = reinterpret_cast<const float4*>(xrow[t])[ic];
+    if (i < n4) {
+      *reinterpret_cast<float4*>(s_nw + xn_at(4 * i)) = nq;
+#pragma unroll
+      for (int t = 0; t < TC; ++t) *reinterpret_cast<float4*>(s_xn + t * kXnPad + xn_at(4 * i)) = xq[t];
+    }
+  }
+  __syncthreads();
+  if (row0 >= n_rows) return;
+  // from here on every wavefront works for itself, out of LDS: the RMS scale of each token in the canonical order
+  // (lane L folds elements 32L .. 32L+31, then the wavefront tree), its own 32 elements normalised as (x * inv) * w
+  auto lds8 = [&](const float* row, int e, float (&v)[32], int at) __attribute__((always_inline)) {
+    const float4* p = reinterpret_cast<const float4*>(row + xn_at(e));
+    const float4 lo = p[0], hi = p[1];
+    v[at + 0] = lo.x; v[at + 1] = lo.y; v[at + 2] = lo.z; v[at + 3] = lo.w;
+    v[at + 4] = hi.x; v[at + 5] = hi.y; v[at + 6] = hi.z; v[at + 7] = hi.w;
+  };
+  float x[TC][32], xs[TC][4], nw[32];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int off = QUANT == kQ6K ? koff + g.half * 128 + j * 32 + g.l8 * 8 : koff + j * 8;
+    lds8(s_nw, off, nw, j * 8);
+#pragma unroll
+    for (int t = 0; t < TC; ++t) lds8(s_xn + t * kXnPad, off, x[t], j * 8);
+  }
 #pragma unroll
   for (int t = 0; t < TC; ++t) {
-    float s = 0.0f;
-    if constexpr (kOwnRms) {
-      s = rms_fold(q[t], 0.0f);
-    } else {
+    float f[32];
+    const int base = g.lane * 32;  // (lanes past the row's end fold zeros: fma(0, 0, s) == s)
 #pragma unroll
-      for (int i = 0; i < 32; ++i) s = __builtin_fmaf(x[t][i], x[t][i], s);
-      if (g.lane * 32 >= K) s = 0.0f;  // lanes past the row's end hold another lane's elements
-    }
-    const float inv = rms_finish(s, K, eps);
+    for (int j = 0; j < 4; ++j) lds8(s_xn + t * kXnPad, min(base, K - 32) + j * 8, f, j * 8);
+    float sq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) sq = __builtin_fmaf(f[i], f[i], sq);
+    if (base >= K) sq = 0.0f;
+    const float inv = rms_finish(sq, K, eps);
 #pragma unroll
     for (int i = 0; i < 32; ++i) x[t][i] = x[t][i] * inv * nw[i];
     lane_x_offsets<QUANT>(x[t], xs[t]);
   }
-  // the live-token count was requested first and is only needed here: rows past it were computed from
-  // whatever the buffer held (in bounds, sized for max_tokens) and are dropped
+  // rows past the live-token count were computed from whatever the buffer held (in bounds, sized for max_tokens)
+  // and are dropped
   const int valid = *valid_tokens;
 #pragma unroll
   for (int d = 0; d < D; ++d) {
@@ -168,6 +205,7 @@ __device__ __forceinline__ void step_normed(const uint8_t* __restrict__ w0, cons
 template <int SQ, int RF, int RPS, int kLogitsDepth>
 __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
   __shared__ float s_red[4];
+  __shared__ __attribute__((aligned(16))) float s_xn[3 * kXnPad];  // the chunk's rows and the norm weight
   const int chunks = (a.max_tokens + 1) / 2;
   const int n_r = chunks * a.tiles_r;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -184,19 +222,19 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
       const float* const xr[2] = {x0, x0 + a.H};
       if (router) {
         float* const o[2] = {a.logits + (size_t)t0 * a.E, a.logits + (size_t)(t0 + 1) * a.E};
-        step_normed<RF, RPS, 2, 1, kLogitsDepth>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0);
+        tile_normed<RF, RPS, 2, 1, kLogitsDepth>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0, s_xn);
       } else {
         float* const o[2] = {a.shared_inter + (size_t)t0 * a.I, a.shared_inter + (size_t)(t0 + 1) * a.I};
-        step_normed<SQ, RPS, 2, 2, kLogitsDepth>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0);
+        tile_normed<SQ, RPS, 2, 2, kLogitsDepth>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0, s_xn);
       }
     } else {
       const float* const xr[1] = {x0};
       if (router) {
         float* const o[1] = {a.logits + (size_t)t0 * a.E};
-        step_normed<RF, RPS, 1, 1, kLogitsDepth>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0);
+        tile_normed<RF, RPS, 1, 1, kLogitsDepth>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0, s_xn);
       } else {
         float* const o[1] = {a.shared_inter + (size_t)t0 * a.I};
-        step_normed<SQ, RPS, 1, 2, kLogitsDepth>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0);
+        tile_normed<SQ, RPS, 1, 2, kLogitsDepth>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0, s_xn);
       }
     }
     XABE_TRACE(0, 3);
@@ -257,7 +295,12 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   XABE_TRACE(1, 0);
   // one wavefront routes the token (a different one in neighbouring workgroups, which share a CU); its
   // logits and every wavefront's copy of the normalised row are requested together
+#ifdef EXP_B_NO_ROUTE
+  const bool routes = false;
+  if (threadIdx.x == 0) { s_expert = (p * 29 + 5) & 255; s_final = s_expert; }
+#else
   const bool routes = wave == (int)((blockIdx.x >> 8) & 3);
+#endif
   const bool few = a.E <= 256;
   float lg[kRouteMaxPerLane];
   if (routes) {
@@ -265,19 +308,32 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
     else route_load<kRouteMaxPerLane>(a.logits + (size_t)t * a.E, a.E, nullptr, nullptr, lg);
   }
   float x[1][32], xs[1][4];
+#ifdef EXP_B_NOX
+#pragma unroll
+  for (int i = 0; i < 32; ++i) x[0][i] = 0.01f * (float)(i + t + g.lane);
+#else
   lane_x_load<RQ>(a.normed + (size_t)t * a.H, koff, g, x[0]);
+#endif
   if (t >= valid) return;
   // Routing in two halves (route_device.h).  The first orders the experts by logit: its k-th candidate is
   // the pair's expert unless probabilities tie, and it is known ~2 us before the softmax is, so the four
   // wavefronts request the candidate's rows right away.  The routing wavefront then finishes the softmax
   // under its own loads' latency; in the rare pass where the probabilities reorder the candidates, the rows
   // are streamed again for the expert the reference's rule selects.
+  // The pair's candidate is known after k + 1 selection rounds; the remaining rounds (the rest of the token's
+  // selection and the k + 1-th candidate the verification needs) run after the rows have been requested.
   const int n_cand = min(a.top_k + 1, a.E);
   int cand_i = 0;
+  int key[kRouteMaxPerLane];
   if (routes) {
     XABE_ROUTE_TRACE(0);
-    if (few) route_order<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, n_cand, cand_i);
-    else route_order<kRouteMaxPerLane>(lg, a.E, n_cand, cand_i);
+    if (few) {
+      route_keys<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, *reinterpret_cast<int(*)[4]>(key));
+      route_rounds<4>(*reinterpret_cast<int(*)[4]>(key), 0, k + 1, cand_i);
+    } else {
+      route_keys<kRouteMaxPerLane>(lg, a.E, key);
+      route_rounds<kRouteMaxPerLane>(key, 0, k + 1, cand_i);
+    }
     if (g.lane == k) s_expert = cand_i;
   }
   lane_x_offsets<RQ>(x[0], xs[0]);
@@ -310,6 +366,8 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
         int sel_i;
         float sel_w;
         bool exact;
+        if (few) route_rounds<4>(*reinterpret_cast<int(*)[4]>(key), k + 1, n_cand, cand_i);
+        else route_rounds<kRouteMaxPerLane>(key, k + 1, n_cand, cand_i);
         if (few) route_finish<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, a.top_k, n_cand, cand_i, s_route, sel_i, sel_w, exact);
         else route_finish<kRouteMaxPerLane>(lg, a.E, a.top_k, n_cand, cand_i, s_route, sel_i, sel_w, exact);
         XABE_ROUTE_TRACE(5);
@@ -321,7 +379,44 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
         __builtin_amdgcn_s_setprio(0);
       }
     }
+#if defined(EXP_B_COALESCED)
+    {
+      // timing only: the wave's 2 x DEPTH rows as consecutive 16-byte pieces
+      const size_t nb = (size_t)DEPTH * RPS * row_bytes;  // bytes per matrix for this wave (multiple of 16: 6720)
+      const uint4* pg = reinterpret_cast<const uint4*>(wg + (size_t)wave_row0 * row_bytes);
+      const uint4* pu = reinterpret_cast<const uint4*>(wu + (size_t)wave_row0 * row_bytes);
+      const int n16 = (int)(nb / 16);
+      uint4 acc4 = make_uint4(0, 0, 0, 0);
+      uint4 v[14];
+#pragma unroll
+      for (int i = 0; i < 7; ++i) {
+        const int j = min(g.lane + 64 * i, n16 - 1);
+        v[i] = pg[j];
+        v[7 + i] = pu[j];
+      }
+#pragma unroll
+      for (int i = 0; i < 14; ++i) { acc4.x ^= v[i].x; acc4.y ^= v[i].y; acc4.z ^= v[i].z; acc4.w ^= v[i].w; }
+      if ((acc4.x ^ acc4.y ^ acc4.z ^ acc4.w) == 0x9e3779b9u + (uint32_t)g.lane) out[wave_row0] = x[0][0];  // (every lane's data is live)
+      return;
+    }
+#endif
     request(0, DEPTH);  // (the other wavefronts come straight here)
+#if defined(EXP_B_NOCOMPUTE)
+    {
+      uint32_t z = 0;
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          uint32_t w[sizeof(Raw) / 4];
+          __builtin_memcpy(w, &r[d][m], sizeof(Raw));
+#pragma unroll
+          for (unsigned i = 0; i < sizeof(Raw) / 4; ++i) z ^= w[i];
+        }
+      if (z == 0x9e3779b9u + (uint32_t)g.lane) out[wave_row0] = x[0][0];  // (every lane's data is live)
+      return;
+    }
+#endif
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (d == 1) XABE_TRACE(1, 2);
@@ -342,90 +437,143 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// C: grid = max_tokens * tiles_d.  A tile is 4 wavefronts x RPS rows; K = intermediate = 2048 / RPS.
+// C: grid = max_tokens * tiles_d.  A workgroup is RS row steps (RPS rows each; K = intermediate = 2048 / RPS)
+// x two wavefronts per step: the first takes the first half of the token's selections and the shared expert,
+// the second the other half, so that a token's nine contractions per row step spread over twice as many
+// wavefronts and every SIMD of the chip gets the same number of them (max_tokens x hidden / RPS x 2
+// wavefronts: 12 per CU at three tokens).  The second wavefront hands its weighted row sums to the first
+// through LDS, which adds all of them in selection order: the same operations as one wavefront would do.
 // ------------------------------------------------------------------------------------------------
-template <int RQ, int SQ, int RPS>
-__global__ void __launch_bounds__(256) k_decode_down(DecodeArgs a) {
+template <int RQ, int SQ, int RPS, int RS>
+__global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
   using RawR = typename Fmt<RQ>::Raw;
   using RawS = typename Fmt<SQ>::Raw;
   constexpr int G = 64 / RPS;
+  constexpr int kThreads = 128 * RS;
+  constexpr int kHalf = kMaxTopK / 2;  // selections per wavefront
   __shared__ __attribute__((aligned(16))) float s_x[(kMaxTopK + 1) * kMaxInter];
+  __shared__ float s_xs[(kMaxTopK + 1) * kMaxInter / 8];  // -32 * (sum of each run of eight), Q6_K's code offset
+  __shared__ float s_part[RS][kHalf][RPS];               // the second wavefront's weighted row sums
   const int t = blockIdx.x / a.tiles_d, tile = blockIdx.x % a.tiles_d;
   // every buffer read below is sized for max_tokens rows, so round one is issued before the live-token
   // count is known; rows past it hold an earlier pass's values or zeros, and nothing is stored for them
   const int valid = *a.valid_tokens;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int rs = wave >> 1, second = wave & 1;
   const int lane = __lane_id();
-  const int row0 = (tile * kWavesPerWg + wave) * RPS;  // hidden is a multiple of 4 * RPS
+  const int row0 = (tile * RS + rs) * RPS;  // hidden is a multiple of RS * RPS
   XABE_TRACE(2, 0);
-  // round one: selections, gate scalar, the nine activation rows (into LDS), the shared expert's rows
-  int my_e = 0;
-  float my_w = 0.0f;
-  if (lane < a.top_k) {
-    my_e = a.topk_ids[(size_t)t * a.top_k + lane];
-    my_w = a.topk_weights[(size_t)t * a.top_k + lane];
+  // this wavefront's selections: [k0, k1)
+  const int split = (a.top_k + 1) / 2;
+  const int k0 = second ? split : 0, k1 = second ? a.top_k : split;
+  // round one: selections (addressed uniformly, so they come through the scalar cache and arrive in the registers
+  // the row addresses are formed from), gate scalar, the nine activation rows, the shared expert's rows
+  int sel_e[kHalf];
+  float sel_w[kHalf];
+#pragma unroll
+  for (int j = 0; j < kHalf; ++j) {
+    const int kk = min(k0 + j, a.top_k - 1);
+    sel_e[j] = a.topk_ids[(size_t)t * a.top_k + kk];
+    sel_w[j] = a.topk_weights[(size_t)t * a.top_k + kk];
   }
   const float gate = a.gate_out[t];
-  constexpr int kStage = ((kMaxTopK + 1) * kMaxInter / 4 + 255) / 256;  // float4 per thread
-  float4 stage[kStage];
-  const int n4 = a.I / 4;
+  // a thread stages whole runs of eight consecutive activations (two 16-byte pieces): the run's sum is then
+  // formed once per workgroup, in element order, instead of once per lane and selection
+  constexpr int kRunsMax = (kMaxTopK + 1) * kMaxInter / 8;
+  constexpr int kStage = (kRunsMax + kThreads - 1) / kThreads;
+  float4 stage[kStage][2];
+  const int runs_per_row = a.I / 8, n_runs = (a.top_k + 1) * runs_per_row;
   {
     const float4* src_r = reinterpret_cast<const float4*>(a.inter + (size_t)t * a.top_k * a.I);
     const float4* src_s = reinterpret_cast<const float4*>(a.shared_inter + (size_t)t * a.I);
 #pragma unroll
     for (int j = 0; j < kStage; ++j) {
-      const int i = threadIdx.x + 256 * j;
-      stage[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (i < (a.top_k + 1) * n4) stage[j] = i < a.top_k * n4 ? src_r[i] : src_s[i - a.top_k * n4];
+      const int i = threadIdx.x + kThreads * j;
+      stage[j][0] = stage[j][1] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < n_runs) {
+        const float4* p = i < a.top_k * runs_per_row ? src_r + 2 * i : src_s + 2 * (i - a.top_k * runs_per_row);
+        stage[j][0] = p[0];
+        stage[j][1] = p[1];
+      }
     }
   }
   const LaneGeom gs = lane_geom<SQ>();
   const LaneGeom gr = lane_geom<RQ>();
   const size_t rb_s = (size_t)(a.I / Fmt<SQ>::kBlockElems) * Fmt<SQ>::kBlockBytes;
   const size_t rb_r = (size_t)(a.I / Fmt<RQ>::kBlockElems) * Fmt<RQ>::kBlockBytes;
-  RawS rs;
-  load_raw<SQ, true>(a.sdown + (size_t)row0 * rb_s, true, gs, rs);
+  RawS raw_s;
+  if (!second) load_raw<SQ, true>(a.sdown + (size_t)row0 * rb_s, true, gs, raw_s);
   if (t >= valid) return;
   // round two: the selected experts' rows
-  RawR rr[kMaxTopK];
+  RawR rr[kHalf];
 #pragma unroll
-  for (int k = 0; k < kMaxTopK; ++k) {
-    const int e = min(max(__builtin_amdgcn_readlane(my_e, k), 0), a.E - 1);
-    // k >= top_k reads expert 0's rows and never uses them: an unconditional load keeps all of round two
-    // in one basic block, so every load is issued before the first wait
-    load_raw<RQ, true>(a.down + (size_t)e * a.down_bytes + (size_t)row0 * rb_r, true, gr, rr[k]);
+  for (int j = 0; j < kHalf; ++j) {
+    const int e = min(max(sel_e[j], 0), a.E - 1);
+    // j past this wavefront's share reads a selected expert's rows again and never uses them: an unconditional
+    // load keeps all of round two in one basic block, so every load is issued before the first wait
+    load_raw<RQ, true>(a.down + (size_t)e * a.down_bytes + (size_t)row0 * rb_r, true, gr, rr[j]);
   }
-  // the activation rows arrived before the weights (loads return in order); publish them to LDS
+  // the activation rows arrived before the weights (loads return in order); publish them and their run sums
 #pragma unroll
   for (int j = 0; j < kStage; ++j) {
-    const int i = threadIdx.x + 256 * j;
-    if (i < (a.top_k + 1) * n4) reinterpret_cast<float4*>(s_x)[i] = stage[j];
+    const int i = threadIdx.x + kThreads * j;
+    if (i < n_runs) {
+      reinterpret_cast<float4*>(s_x)[2 * i] = stage[j][0];
+      reinterpret_cast<float4*>(s_x)[2 * i + 1] = stage[j][1];
+      float sum = 0.0f;  // (the order of lane_x_offsets)
+      sum += stage[j][0].x; sum += stage[j][0].y; sum += stage[j][0].z; sum += stage[j][0].w;
+      sum += stage[j][1].x; sum += stage[j][1].y; sum += stage[j][1].z; sum += stage[j][1].w;
+      s_xs[i] = -32.0f * sum;
+    }
   }
   __syncthreads();
   XABE_TRACE(2, 1);
-  float r = 0.0f;
+  // x[32] of one staged row for this lane, and (Q6_K) the four run sums that go with them
+  auto lane_x = [&](auto quant_c, int slot, const LaneGeom& g, float (&x)[1][32], float (&xs)[1][4]) __attribute__((always_inline)) {
+    constexpr int Q = decltype(quant_c)::value;
+    const int koff = lane_koff<Q, RPS>(g, 0);
+    lane_x_load<Q>(s_x + slot * a.I, koff, g, x[0]);
 #pragma unroll
-  for (int k = 0; k < kMaxTopK; ++k) {
-    if (k < a.top_k) {
+    for (int j = 0; j < 4; ++j)
+      xs[0][j] = Q == kQ6K ? s_xs[slot * runs_per_row + (koff + g.half * 128 + j * 32 + g.l8 * 8) / 8] : 0.0f;
+  };
+  float part[kHalf];
+#pragma unroll
+  for (int j = 0; j < kHalf; ++j) {
+    part[j] = 0.0f;
+    if (k0 + j < k1) {
       float x[1][32], xs[1][4], tot[1] = {0.0f};
-      lane_x_load<RQ>(s_x + k * a.I, lane_koff<RQ, RPS>(gr, 0), gr, x[0]);
-      lane_x_offsets<RQ>(x[0], xs[0]);
-      accum<RQ, 1>(rr[k], gr, x, xs, tot);
-      const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_w), k));
-      r += w * group_sum<G>(tot[0]);
+      lane_x(std::integral_constant<int, RQ>{}, k0 + j, gr, x, xs);
+      accum<RQ, 1>(rr[j], gr, x, xs, tot);
+      part[j] = sel_w[j] * group_sum<G>(tot[0]);
     }
   }
   XABE_TRACE(2, 2);
-  float sh;
-  {
+  const bool writes = (lane % G) == 0;
+  if (second) {
+    if (writes) {
+#pragma unroll
+      for (int j = 0; j < kHalf; ++j) s_part[rs][j][lane / G] = part[j];
+    }
+  }
+  float sh = 0.0f;
+  if (!second) {
     float x[1][32], xs[1][4], tot[1] = {0.0f};
-    lane_x_load<SQ>(s_x + a.top_k * a.I, lane_koff<SQ, RPS>(gs, 0), gs, x[0]);
-    lane_x_offsets<SQ>(x[0], xs[0]);
-    accum<SQ, 1>(rs, gs, x, xs, tot);
+    lane_x(std::integral_constant<int, SQ>{}, a.top_k, gs, x, xs);
+    accum<SQ, 1>(raw_s, gs, x, xs, tot);
     sh = 1.0f * group_sum<G>(tot[0]);
   }
+  __syncthreads();
   const int row = row0 + lane / G;
-  if ((lane % G) == 0 && row < a.H) {
+  if (!second && writes && row < a.H) {
+    // the routed sum in selection order: this wavefront's share, then the other's
+    float r = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kHalf; ++j)
+      if (j < k1) r += part[j];
+#pragma unroll
+    for (int j = 0; j < kHalf; ++j)
+      if (split + j < a.top_k) r += s_part[rs][j][lane / G];
     const size_t i = (size_t)t * a.H + row;
     const float v = r + sh * gate;
     a.routed[i] = r;
@@ -472,7 +620,10 @@ static bool launch_all(const Launch& l, int gq, int dq, int sgq, int sdq, int ro
     else hipLaunchKernelGGL((k_decode_up<kQ8_0, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
   }
   if (l.launches & 4u) {
-#define XABE_C(RQ, SQ) hipLaunchKernelGGL((k_decode_down<RQ, SQ, RPSI>), dim3(l.grid_c), dim3(256), 0, l.s, l.a)
+#define XABE_C(RQ, SQ)                                                                                            \
+  do {                                                                                                          \
+    hipLaunchKernelGGL((k_decode_down<RQ, SQ, RPSI, kDownSteps>), dim3(l.grid_c), dim3(128 * kDownSteps), 0, l.s, l.a); \
+  } while (0)
     if (d6 && sd6) XABE_C(kQ6K, kQ6K);
     else if (d6) XABE_C(kQ6K, kQ8_0);
     else if (sd6) XABE_C(kQ8_0, kQ6K);
@@ -544,8 +695,9 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
   a.tiles_s = (a.I + kWavesPerWg * rps_h * da - 1) / (kWavesPerWg * rps_h * da);
   const int depth = a.H == 2048 ? 4 : 1;  // steps per wavefront of the gate/up launch (launch_shape)
   a.tiles_g = (a.I + kWavesPerWg * depth * rps_h - 1) / (kWavesPerWg * depth * rps_h);
-  a.tiles_d = (a.H + kWavesPerWg * rps_i - 1) / (kWavesPerWg * rps_i);
-  if (a.E % rps_h != 0 || a.I % (kWavesPerWg * depth * rps_h) != 0 || a.H % (kWavesPerWg * rps_i) != 0)
+  const int down_steps = kDownSteps;
+  a.tiles_d = (a.H + down_steps * rps_i - 1) / (down_steps * rps_i);
+  if (a.E % rps_h != 0 || a.I % (kWavesPerWg * depth * rps_h) != 0 || a.H % (down_steps * rps_i) != 0)
     return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "decode block: %d experts / %d intermediate rows do not fill whole steps of %d rows",
                      a.E, a.I, rps_h);
   const int chunks = (a.max_tokens + 1) / 2;

@@ -40,6 +40,9 @@ __device__ __forceinline__ void route_load(const float* lg, int num_experts, con
 
 // One selection round over per-lane keys (kTaken = out of the running): the largest key, the lowest index
 // among equals; the winner is marked taken.  Returns the winning key and index to every lane.
+// Almost always exactly one (lane, slot) holds the maximum: then its index is read straight off the ballots and
+// every holder (the one) is retired.  Several holders (equal keys) take the general path, which finds the lowest
+// index among them and retires that one alone.
 constexpr int kRouteTaken = (int)0x80000000;
 template <int PER>
 __device__ __forceinline__ void route_round(int (&key)[PER], int& best, int& bi) {
@@ -48,13 +51,27 @@ __device__ __forceinline__ void route_round(int (&key)[PER], int& best, int& bi)
 #pragma unroll
   for (int i = 1; i < PER; ++i) bp = max(bp, key[i]);
   best = wave_max_i(bp);
+  unsigned long long holders[PER];
+  int n_holders = 0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    holders[i] = __builtin_amdgcn_ballot_w64(key[i] == best);
+    n_holders += __builtin_popcountll(holders[i]);
+  }
+  if (n_holders == 1) {  // (wave-uniform)
+    bi = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (holders[i]) bi = i * 64 + __builtin_ctzll(holders[i]);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) key[i] = key[i] == best ? kRouteTaken : key[i];
+    return;
+  }
   int li = 0x7fffffff;
 #pragma unroll
   for (int i = PER - 1; i >= 0; --i)
     if (key[i] == best) li = i * 64 + lane;  // descending i: the lowest index of this lane wins
-  const unsigned long long holders = __builtin_amdgcn_ballot_w64(li != 0x7fffffff);
-  if (__builtin_popcountll(holders) == 1) bi = __builtin_amdgcn_readlane(li, __builtin_ctzll(holders));
-  else bi = wave_min_i(li);
+  bi = wave_min_i(li);
   if ((bi & 63) == lane) {
 #pragma unroll
     for (int i = 0; i < PER; ++i)
@@ -67,21 +84,32 @@ __device__ __forceinline__ void route_round(int (&key)[PER], int& best, int& bi)
 // monotone non-decreasing, so p orders the experts the same way except where distinct logits round to the
 // same p: with n = top_k + 1 candidates, route_finish sees whether that happened anywhere it matters, and
 // the candidates are then the selection itself -- known before a single exp has been evaluated.
+// In two steps so that a caller who needs the j-th candidate only can act on it after j + 1 rounds:
+// route_keys makes the keys, route_rounds runs rounds [j0, j1) and leaves the j-th winner in lane j's cand_i.
 template <int PER>
-__device__ __forceinline__ void route_order(const float (&l)[PER], int num_experts, int n, int& cand_i) {
+__device__ __forceinline__ void route_keys(const float (&l)[PER], int num_experts, int (&key)[PER]) {
   const int lane = threadIdx.x & 63;
-  int key[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int b = __builtin_bit_cast(int, l[i]);
     key[i] = i * 64 + lane < num_experts ? b ^ ((b >> 31) & 0x7fffffff) : kRouteTaken;  // int order == float order
   }
-  cand_i = 0;
-  for (int j = 0; j < n; ++j) {
+}
+template <int PER>
+__device__ __forceinline__ void route_rounds(int (&key)[PER], int j0, int j1, int& cand_i) {
+  const int lane = threadIdx.x & 63;
+  for (int j = j0; j < j1; ++j) {
     int best, bi;
     route_round<PER>(key, best, bi);
     if (lane == j) cand_i = bi;
   }
+}
+template <int PER>
+__device__ __forceinline__ void route_order(const float (&l)[PER], int num_experts, int n, int& cand_i) {
+  int key[PER];
+  route_keys<PER>(l, num_experts, key);
+  cand_i = 0;
+  route_rounds<PER>(key, 0, n, cand_i);
 }
 
 // Second half: softmax, then the selection.  If the top_k + 1 candidates' probabilities are strictly
