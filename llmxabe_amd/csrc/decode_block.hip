@@ -38,6 +38,12 @@ namespace xabe { static __device__ long long g_route_trace[4096 * 8]; }
 namespace xabe {
 
 constexpr size_t kDecodeBlockMaxTokens = 32;  // widest batch served by the three launches (at 32 tokens 198 against the dispatch-table regime's 203 us; it wins beyond)
+// From this width on the routing is a launch of its own between the first two (one wavefront per token) and the second
+// launch reads the selections: inside the second launch every workgroup of a token repeats the token's routing, and
+// past a few tokens its grid runs in several rounds per CU, each paying for it again.  Same-box, us per block, routing
+// inside / routing launch: 4 tokens 38.6 / 40.5, 6: 49.8 / 51.2, 8: 61.5 / 61.1, 12: 83.3 / 79.4, 16: 101.7 / 94.9,
+// 32: 181.3 / 161.5.
+constexpr int kPreRouteMinTokens = 8;
 constexpr int kMaxTopK = 8;       // contributions held in registers by k_decode_down
 constexpr int kMaxInter = 512;    // intermediate width staged in LDS by k_decode_down
 // Steps per wavefront of the first launch: a wavefront reads 24 KB of activation rows and norm weights for the 2-4 KB
@@ -278,7 +284,25 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
 // ------------------------------------------------------------------------------------------------
 // B: grid = max_tokens * top_k * tiles_g.  A tile is 4 wavefronts x DEPTH steps x RPS rows.
 // ------------------------------------------------------------------------------------------------
-template <int RQ, int RPS, int DEPTH>
+// The routing launch of wider batches: one wavefront per token (route_one_token, the stand-alone routing kernel's
+// body), one token per workgroup so that the tokens spread over the chip.
+__global__ void __launch_bounds__(64) k_decode_route(DecodeArgs a) {
+  extern __shared__ float s_route_one[];  // num_experts floats
+  const int t = blockIdx.x;
+  if (t >= *a.valid_tokens) return;
+  int sel_i;
+  float sel_w;
+  route_one_token(a.logits + (size_t)t * a.E, a.E, a.top_k, s_route_one, sel_i, sel_w);
+  if ((int)threadIdx.x < a.top_k) {
+    a.topk_ids[(size_t)t * a.top_k + threadIdx.x] = sel_i;
+    a.topk_weights[(size_t)t * a.top_k + threadIdx.x] = sel_w;
+  }
+}
+
+// ROUTED: the token's selection was made by a routing launch between A and this one (wider batches: there a token's
+// routing would otherwise be repeated by every one of its workgroups, several rounds of them per CU); the pair's
+// expert then comes out of topk_ids through the scalar cache and nothing else of the routing runs here.
+template <int RQ, int RPS, int DEPTH, bool ROUTED = false>
 __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   using F = Fmt<RQ>;
   using Raw = typename F::Raw;
@@ -287,6 +311,8 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   __shared__ int s_expert, s_final;  // the candidate expert of this pair; the one routing settles on
   const int p = blockIdx.x / a.tiles_g, tile = blockIdx.x % a.tiles_g;
   const int t = p / a.top_k, k = p % a.top_k;
+  [[maybe_unused]] int pre_e = 0;
+  if constexpr (ROUTED) pre_e = a.topk_ids[p];
   // everything read before the live-token count is known is sized for max_tokens rows
   const int valid = *a.valid_tokens;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -295,12 +321,7 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   XABE_TRACE(1, 0);
   // one wavefront routes the token (a different one in neighbouring workgroups, which share a CU); its
   // logits and every wavefront's copy of the normalised row are requested together
-#ifdef EXP_B_NO_ROUTE
-  const bool routes = false;
-  if (threadIdx.x == 0) { s_expert = (p * 29 + 5) & 255; s_final = s_expert; }
-#else
-  const bool routes = wave == (int)((blockIdx.x >> 8) & 3);
-#endif
+  const bool routes = !ROUTED && wave == (int)((blockIdx.x >> 8) & 3);
   const bool few = a.E <= 256;
   float lg[kRouteMaxPerLane];
   if (routes) {
@@ -308,12 +329,7 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
     else route_load<kRouteMaxPerLane>(a.logits + (size_t)t * a.E, a.E, nullptr, nullptr, lg);
   }
   float x[1][32], xs[1][4];
-#ifdef EXP_B_NOX
-#pragma unroll
-  for (int i = 0; i < 32; ++i) x[0][i] = 0.01f * (float)(i + t + g.lane);
-#else
   lane_x_load<RQ>(a.normed + (size_t)t * a.H, koff, g, x[0]);
-#endif
   if (t >= valid) return;
   // Routing in two halves (route_device.h).  The first orders the experts by logit: its k-th candidate is
   // the pair's expert unless probabilities tie, and it is known ~2 us before the softmax is, so the four
@@ -337,7 +353,7 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
     if (g.lane == k) s_expert = cand_i;
   }
   lane_x_offsets<RQ>(x[0], xs[0]);
-  __syncthreads();
+  if constexpr (!ROUTED) __syncthreads();
   XABE_TRACE(1, 1);
   const size_t row_bytes = (size_t)(a.H / F::kBlockElems) * F::kBlockBytes;
   const int wave_row0 = (tile * kWavesPerWg + wave) * DEPTH * RPS;
@@ -379,44 +395,7 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
         __builtin_amdgcn_s_setprio(0);
       }
     }
-#if defined(EXP_B_COALESCED)
-    {
-      // timing only: the wave's 2 x DEPTH rows as consecutive 16-byte pieces
-      const size_t nb = (size_t)DEPTH * RPS * row_bytes;  // bytes per matrix for this wave (multiple of 16: 6720)
-      const uint4* pg = reinterpret_cast<const uint4*>(wg + (size_t)wave_row0 * row_bytes);
-      const uint4* pu = reinterpret_cast<const uint4*>(wu + (size_t)wave_row0 * row_bytes);
-      const int n16 = (int)(nb / 16);
-      uint4 acc4 = make_uint4(0, 0, 0, 0);
-      uint4 v[14];
-#pragma unroll
-      for (int i = 0; i < 7; ++i) {
-        const int j = min(g.lane + 64 * i, n16 - 1);
-        v[i] = pg[j];
-        v[7 + i] = pu[j];
-      }
-#pragma unroll
-      for (int i = 0; i < 14; ++i) { acc4.x ^= v[i].x; acc4.y ^= v[i].y; acc4.z ^= v[i].z; acc4.w ^= v[i].w; }
-      if ((acc4.x ^ acc4.y ^ acc4.z ^ acc4.w) == 0x9e3779b9u + (uint32_t)g.lane) out[wave_row0] = x[0][0];  // (every lane's data is live)
-      return;
-    }
-#endif
     request(0, DEPTH);  // (the other wavefronts come straight here)
-#if defined(EXP_B_NOCOMPUTE)
-    {
-      uint32_t z = 0;
-#pragma unroll
-      for (int d = 0; d < DEPTH; ++d)
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-          uint32_t w[sizeof(Raw) / 4];
-          __builtin_memcpy(w, &r[d][m], sizeof(Raw));
-#pragma unroll
-          for (unsigned i = 0; i < sizeof(Raw) / 4; ++i) z ^= w[i];
-        }
-      if (z == 0x9e3779b9u + (uint32_t)g.lane) out[wave_row0] = x[0][0];  // (every lane's data is live)
-      return;
-    }
-#endif
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (d == 1) XABE_TRACE(1, 2);
@@ -428,11 +407,15 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
       if ((g.lane % G) == 0 && row < a.I) out[row] = silu_f(sg) * su;
     }
   };
-  const int e = s_expert;
-  stream_rows(e, std::true_type{});
-  __syncthreads();  // s_final is there
-  const int e_final = s_final;
-  if (e_final != e) stream_rows(e_final, std::false_type{});  // (same rows of `inter`, written again)
+  if constexpr (ROUTED) {
+    stream_rows(min(max(pre_e, 0), a.E - 1), std::false_type{});
+  } else {
+    const int e = s_expert;
+    stream_rows(e, std::true_type{});
+    __syncthreads();  // s_final is there
+    const int e_final = s_final;
+    if (e_final != e) stream_rows(e_final, std::false_type{});  // (same rows of `inter`, written again)
+  }
   XABE_TRACE(1, 3);
 }
 
@@ -589,6 +572,7 @@ struct Launch {
   const DecodeArgs& a;
   hipStream_t s;
   unsigned grid_a, grid_b, grid_c;
+  bool pre_routed;  // a routing launch between A and B instead of routing inside B
   size_t route_lds;
   unsigned launches;  // bit i: issue launch i (A, B, C); all three outside measurements
 };
@@ -616,7 +600,11 @@ static bool launch_all(const Launch& l, int gq, int dq, int sgq, int sdq, int ro
 #undef XABE_A
   }
   if (l.launches & 2u) {
-    if (g6) hipLaunchKernelGGL((k_decode_up<kQ6K, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
+    if (l.pre_routed) {
+      hipLaunchKernelGGL(k_decode_route, dim3((unsigned)l.a.max_tokens), dim3(64), l.route_lds, l.s, l.a);
+      if (g6) hipLaunchKernelGGL((k_decode_up<kQ6K, RPSH, DEPTH, true>), dim3(l.grid_b), dim3(256), 0, l.s, l.a);
+      else hipLaunchKernelGGL((k_decode_up<kQ8_0, RPSH, DEPTH, true>), dim3(l.grid_b), dim3(256), 0, l.s, l.a);
+    } else if (g6) hipLaunchKernelGGL((k_decode_up<kQ6K, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
     else hipLaunchKernelGGL((k_decode_up<kQ8_0, RPSH, DEPTH>), dim3(l.grid_b), dim3(256), l.route_lds, l.s, l.a);
   }
   if (l.launches & 4u) {
@@ -701,7 +689,8 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
     return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "decode block: %d experts / %d intermediate rows do not fill whole steps of %d rows",
                      a.E, a.I, rps_h);
   const int chunks = (a.max_tokens + 1) / 2;
-  Launch l{a, s, 0, 0, 0, g.num_experts * sizeof(float), launches};
+  const bool pre_routed = a.max_tokens >= kPreRouteMinTokens;
+  Launch l{a, s, 0, 0, 0, pre_routed, g.num_experts * sizeof(float), launches};
   l.grid_a = (unsigned)(chunks * (a.tiles_r + a.tiles_s) + a.max_tokens);
   l.grid_b = (unsigned)(a.max_tokens * a.top_k * a.tiles_g);
   l.grid_c = (unsigned)(a.max_tokens * a.tiles_d);

@@ -199,13 +199,9 @@ __device__ __forceinline__ void q6_load_direct(const uint8_t* chunk4, uint32_t l
   r.qb0 = v.x, r.qb1 = v.y;
   __builtin_memcpy(&v, blk + 128 + half * 32 + l8 * 8, 8);
   r.qh0 = v.x, r.qh1 = v.y;
-#ifdef EXP_FEWLOADS
-  r.sc0 = 0x01020304u, r.sc1 = 0x02030401u; r.dh = 0x2000u;
-#else
   __builtin_memcpy(&v, blk + 192 + half * 8, 8);
   r.sc0 = v.x, r.sc1 = v.y;
   r.dh = load_u16(chunk4, lane_off + 208);
-#endif
 }
 
 __device__ __forceinline__ float ub0(uint32_t v) { return (float)(v & 0xffu); }
