@@ -414,6 +414,12 @@ def other_workload(args) -> int:
         width = H
     x = X.synth_normal_f32(99, T * width, 1.0).view(T, width)
     ffn_out, l_out = torch.zeros_like(x), torch.zeros_like(x)
+    if args.calibration_copies:   # a kernel of known traffic for counter runs (see the headline's option)
+        src = torch.zeros(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.calibration_copies):
+            dst.copy_(src)
+        del src, dst
     extra = {}
     if args.workload == "prefill_512":
         # the skewed configuration: a seeded Zipf(s = 1.1) bias over the experts, added to the router logits before

@@ -44,6 +44,18 @@ constexpr size_t kDecodeBlockMaxTokens = 32;  // widest batch served by the thre
 // inside / routing launch: 4 tokens 38.6 / 40.5, 6: 49.8 / 51.2, 8: 61.5 / 61.1, 12: 83.3 / 79.4, 16: 101.7 / 94.9,
 // 32: 181.3 / 161.5.
 constexpr int kPreRouteMinTokens = 8;
+// From this width on the second and third launches deal their workgroups so that the ones that read the same row
+// tile (of whichever experts their pairs or tokens selected) run next to each other on one XCD: workgroup ids go
+// round-robin to the eight XCDs, each with its own L2, and at these widths several pairs select the same expert
+// (32 tokens: 256 pairs over ~163 experts), whose rows then come out of HBM once per XCD instead of once per pair.
+// Fetched per launch at 32 tokens (FETCH_SIZE): gate/up 415 -> 342 MB, down 204 -> 151 MB.  The launches take the
+// same time either way (they are bound by vector instructions at these widths, not by bytes): at 16 tokens and
+// below, where fewer pairs coincide, the plain order measured 0.1-0.5 us faster and is kept.
+// (Grouping the second launch by expert instead, one workgroup per (expert, row tile) running its pairs against
+// one copy of the rows in registers, reads every expert exactly once and was measured slower: 109 us against 95 at
+// 32 tokens with one pair at a time, 135 us two at a time (sharing the dequantisation takes ~230 registers); the
+// pairs of an expert run one after the other there, and a third of the workgroups find no pair at all.)
+constexpr int kXcdGroupMinTokens = 24;
 constexpr int kMaxTopK = 8;       // contributions held in registers by k_decode_down
 constexpr int kMaxInter = 512;    // intermediate width staged in LDS by k_decode_down
 // Steps per wavefront of the first launch: a wavefront reads 24 KB of activation rows and norm weights for the 2-4 KB
@@ -309,7 +321,13 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   constexpr int G = 64 / RPS;
   extern __shared__ float s_route[];  // num_experts floats for the routing wavefront
   __shared__ int s_expert, s_final;  // the candidate expert of this pair; the one routing settles on
-  const int p = blockIdx.x / a.tiles_g, tile = blockIdx.x % a.tiles_g;
+  int p = blockIdx.x / a.tiles_g, tile = blockIdx.x % a.tiles_g;
+  if (ROUTED && a.max_tokens >= kXcdGroupMinTokens && (a.tiles_g & 7) == 0) {
+    // wide batches (see kXcdGroupMinTokens): all pairs of one row tile next to each other on one XCD
+    const int n_pairs = a.max_tokens * a.top_k, xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    tile = xcd + 8 * (j / n_pairs);
+    p = j % n_pairs;
+  }
   const int t = p / a.top_k, k = p % a.top_k;
   [[maybe_unused]] int pre_e = 0;
   if constexpr (ROUTED) pre_e = a.topk_ids[p];
@@ -437,7 +455,13 @@ __global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
   __shared__ __attribute__((aligned(16))) float s_x[(kMaxTopK + 1) * kMaxInter];
   __shared__ float s_xs[(kMaxTopK + 1) * kMaxInter / 8];  // -32 * (sum of each run of eight), Q6_K's code offset
   __shared__ float s_part[RS][kHalf][RPS];               // the second wavefront's weighted row sums
-  const int t = blockIdx.x / a.tiles_d, tile = blockIdx.x % a.tiles_d;
+  int t = blockIdx.x / a.tiles_d, tile = blockIdx.x % a.tiles_d;
+  if (a.max_tokens >= kXcdGroupMinTokens && (a.tiles_d & 7) == 0) {
+    // wide batches (see kXcdGroupMinTokens): all tokens of one row tile next to each other on one XCD
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    tile = xcd + 8 * (j / a.max_tokens);
+    t = j % a.max_tokens;
+  }
   // every buffer read below is sized for max_tokens rows, so round one is issued before the live-token
   // count is known; rows past it hold an earlier pass's values or zeros, and nothing is stored for them
   const int valid = *a.valid_tokens;
