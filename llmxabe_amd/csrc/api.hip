@@ -912,17 +912,39 @@ int xabe_rms_norm(void* stream, const float* x, size_t x_len, const float* weigh
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out)) % 16 != 0)
     return set_error(XABE_ERR_INVALID_ARGUMENT, "rms_norm: x, weight and out must be 16-byte aligned");
   if (width <= 2048 && rows >= 64)  // (a handful of rows: one workgroup per row finishes sooner)
-    hipLaunchKernelGGL(k_rms_norm_short_rows, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, as_stream(stream), x, weight, out,
-                       (int)rows, (int)width, eps);
+    hipLaunchKernelGGL(k_rms_norm_short_rows<false>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, as_stream(stream), x, weight, out,
+                       static_cast<_Float16*>(nullptr), (int)rows, (int)width, eps);
   else
     hipLaunchKernelGGL(k_rms_norm_rows, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), x, weight, out, (int)width, eps);
   XABE_HIP_TRY(hipGetLastError());
   return XABE_OK;
 }
 
+int xabe::rms_norm_rows_with_f16(void* stream, const float* x, const float* weight, float* out, void* out_h, size_t rows,
+                                 size_t width, float eps, bool* done) {
+  *done = false;
+  if (!out_h || width > 2048 || width % 4 != 0 || rows < 64) return XABE_OK;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out) |
+       reinterpret_cast<uintptr_t>(out_h)) % 16 != 0)
+    return XABE_OK;
+  hipLaunchKernelGGL(k_rms_norm_short_rows<true>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, as_stream(stream), x, weight, out,
+                     static_cast<_Float16*>(out_h), (int)rows, (int)width, eps);
+  XABE_HIP_TRY(hipGetLastError());
+  *done = true;
+  return XABE_OK;
+}
+
 int xabe_moe_router_logits(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b, const void* router,
                            size_t router_len, int router_quant, const float* normed, size_t normed_len, float* logits,
                            size_t logits_len) {
+  return router_logits_biased(k, stream, b, router, router_len, router_quant, normed, normed_len, logits, logits_len, nullptr,
+                              nullptr);
+}
+
+int xabe::router_logits_biased(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b, const void* router,
+                               size_t router_len, int router_quant, const float* normed, size_t normed_len, float* logits,
+                               size_t logits_len, const float* bias, bool* bias_added) {
+  if (bias_added) *bias_added = false;
   if (!k || !b || !router || !normed || !logits) return set_error(XABE_ERR_INVALID_ARGUMENT, "router_logits: null pointer");
   const xabe_moe_geometry& g = k->g;
   const size_t elems = g.num_experts * g.hidden;
@@ -940,7 +962,8 @@ int xabe_moe_router_logits(const xabe_moe_kernels* k, void* stream, const xabe_m
   }
   XABE_TRY(check_len("normed", g.max_tokens * g.hidden, normed_len));
   XABE_TRY(check_len("logits", g.max_tokens * g.num_experts, logits_len));
-  if (router_gemm_supported(k, b, fmt)) return launch_router_gemm(k, as_stream(stream), b, router, fmt, normed, logits);
+  if (router_gemm_supported(k, b, fmt))
+    return launch_router_gemm(k, as_stream(stream), b, router, fmt, normed, logits, bias, bias_added);
   ExpertArgs a = base_args(k, b);
   a.w0 = static_cast<const uint8_t*>(router);
   a.x = normed;

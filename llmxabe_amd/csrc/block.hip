@@ -102,9 +102,16 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
                                blk->logits, blk->shexp, blk->gate, blk->routed, ffn_out, l_out);
   }
 
-  // 1. post-mixer RMSNorm over every row of the buffer
-  XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
-                         g.hidden, blk->eps));
+  const bool wide = g.max_tokens >= kMfmaMinTokens && xabe_moe_kernels_tensor_cores_enabled(blk->moe);
+  // 1. post-mixer RMSNorm over every row of the buffer; at matrix-core widths the same launch writes the fp16 copy
+  //    of the rows that the routed and the shared expert kernels read
+  bool normed_h = false;
+  if (wide && blk->buffers->x_h)
+    XABE_TRY(rms_norm_rows_with_f16(stream, residual, w->post_norm, blk->normed, blk->buffers->x_h, g.max_tokens, g.hidden,
+                                    blk->eps, &normed_h));
+  if (!normed_h)
+    XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
+                           g.hidden, blk->eps));
   // 2. router logits, (bias,) softmax + top-k + renormalise, dispatch tables
   if (!(w->router_quant < 0 || w->router_quant == XABE_QUANT_Q8_0))
     return set_error(XABE_ERR_UNSUPPORTED_QUANT, "router: only f32 and Q8_0 routers are supported, got code %d", w->router_quant);
@@ -112,13 +119,13 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
                                 ? g.num_experts * g.hidden
                                 : g.num_experts * g.hidden / xabe_expert_quant_block_elements(w->router_quant) *
                                       xabe_expert_quant_block_bytes(w->router_quant);
-  XABE_TRY(xabe_moe_router_logits(blk->moe, stream, blk->buffers, w->router, router_len, w->router_quant, blk->normed,
-                                  blk->n_act, blk->logits, blk->n_logits));
-  if (logit_bias) XABE_TRY(xabe_moe_add_logit_bias(blk->moe, stream, blk->buffers, logit_bias, blk->logits));
+  bool bias_added = false;
+  XABE_TRY(router_logits_biased(blk->moe, stream, blk->buffers, w->router, router_len, w->router_quant, blk->normed,
+                                blk->n_act, blk->logits, blk->n_logits, logit_bias, &bias_added));
+  if (logit_bias && !bias_added) XABE_TRY(xabe_moe_add_logit_bias(blk->moe, stream, blk->buffers, logit_bias, blk->logits));
   XABE_TRY(xabe_moe_route_and_dispatch(blk->moe, stream, blk->buffers, blk->logits, blk->n_logits));
   // 3 + 4. routed experts (stopping at `partial`) and the ungated shared expert
   int fused = 0;
-  const bool wide = g.max_tokens >= kMfmaMinTokens && xabe_moe_kernels_tensor_cores_enabled(blk->moe);
   if (!wide)
     XABE_TRY(xabe_moe_grouped_forward_partial_with_shared(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps,
                                                           w->down_exps, w->shared_gate, w->shared_up, w->shared_down,
@@ -127,7 +134,9 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
     const bool shared_mma =
         wide && mfma_supported(blk->moe, blk->buffers, w->shared_gate.quant, w->shared_up.quant, w->shared_down.quant, false);
     // the routed and the shared matrix-core paths read the same fp16 copy of the rows: made once here
-    if (shared_mma) {
+    if (normed_h) {
+      blk->buffers->x_h_ready = true;
+    } else if (shared_mma) {
       XABE_TRY(mfma_convert_activations(blk->moe, as_stream(stream), blk->buffers, blk->normed));
       blk->buffers->x_h_ready = true;
     }

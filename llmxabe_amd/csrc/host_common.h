@@ -83,7 +83,17 @@ inline int router_gemm_splits(const xabe_moe_geometry& g) {
 }
 bool router_gemm_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int router_quant);
 int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,
-                       int router_quant, const float* normed, float* logits);
+                       int router_quant, const float* normed, float* logits, const float* bias = nullptr,
+                       bool* bias_added = nullptr);
+// Router logits with the per-expert bias folded into the launch that finishes them where there is one (the split
+// matrix-instruction GEMM's plane sum); `*bias_added` says whether it was (otherwise the caller adds it).
+int router_logits_biased(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b, const void* router,
+                         size_t router_len, int router_quant, const float* normed, size_t normed_len, float* logits,
+                         size_t logits_len, const float* bias, bool* bias_added);
+// RMSNorm of `rows` rows that also writes the fp16 copy the matrix-core kernels read (rows of at most 2048
+// elements, at least 64 of them); returns false in *done when the shape is not served.
+int rms_norm_rows_with_f16(void* stream, const float* x, const float* weight, float* out, void* out_h, size_t rows,
+                           size_t width, float eps, bool* done);
 // one-time, at handle creation: LDS limits of the kernels that ask for more than the static 64 KB (mfma.hip, api.hip)
 int mfma_configure();
 int long_rows_configure();

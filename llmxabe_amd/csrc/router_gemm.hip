@@ -119,13 +119,16 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
   }
 }
 
-// logits[t][e] = planes[0][t][e] + planes[1][t][e] + ... in part order, live tokens only
+// logits[t][e] = planes[0][t][e] + planes[1][t][e] + ... in part order, live tokens only; then (+ bias[e]): the
+// add of the stand-alone bias kernel, on the finished sum
 __global__ void __launch_bounds__(256) k_router_sum_planes(const float* __restrict__ planes, const int* __restrict__ valid_tokens,
-                                                            int splits, int max_tokens, int E, float* __restrict__ logits) {
+                                                            int splits, int max_tokens, int E, const float* __restrict__ bias,
+                                                            float* __restrict__ logits) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= (size_t)*valid_tokens * E) return;
   float s = planes[i];
   for (int z = 1; z < splits; ++z) s += planes[(size_t)z * max_tokens * E + i];
+  if (bias) s += bias[i % (size_t)E];
   logits[i] = s;
 }
 
@@ -142,7 +145,8 @@ bool router_gemm_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b,
 }
 
 int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,
-                       int router_quant, const float* normed, float* logits) {
+                       int router_quant, const float* normed, float* logits, const float* bias, bool* bias_added) {
+  if (bias_added) *bias_added = false;
   const xabe_moe_geometry& g = k->g;
   RouterGemmArgs a;
   memset(&a, 0, sizeof(a));
@@ -161,8 +165,9 @@ int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_
   if (a.splits > 1) {
     const size_t n = g.max_tokens * g.num_experts;
     hipLaunchKernelGGL(k_router_sum_planes, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, b->router_partial,
-                       b->valid_tokens, a.splits, a.max_tokens, a.E, logits);
+                       b->valid_tokens, a.splits, a.max_tokens, a.E, bias, logits);
     XABE_HIP_TRY(hipGetLastError());
+    if (bias && bias_added) *bias_added = true;
   }
   return XABE_OK;
 }

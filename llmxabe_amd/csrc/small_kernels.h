@@ -57,8 +57,12 @@ __global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__
 
 // Rows of at most 2048 elements: one wavefront per row, four rows per workgroup.  The lane's 32 elements
 // are the ones rms_fold takes from it, so the row is read once and normalised out of the same registers.
+// WITH_H: the row also goes out as fp16 (the copy the matrix-core kernels read: the fp32 value rounded once, what
+// the stand-alone conversion kernel writes).
+template <bool WITH_H>
 __global__ void __launch_bounds__(256) k_rms_norm_short_rows(const float* __restrict__ x, const float* __restrict__ w,
-                                                              float* __restrict__ out, int rows, int width, float eps) {
+                                                              float* __restrict__ out, _Float16* __restrict__ out_h, int rows,
+                                                              int width, float eps) {
   const int row = blockIdx.x * 4 + (int)(threadIdx.x >> 6);
   if (row >= rows) return;
   const float* xr = x + (size_t)row * width;
@@ -68,10 +72,18 @@ __global__ void __launch_bounds__(256) k_rms_norm_short_rows(const float* __rest
   const float inv = rms_finish(rms_fold(r, 0.0f), width, eps);
   const int base = (int)__lane_id() * 32;
   float4* o4 = reinterpret_cast<float4*>(out + (size_t)row * width + base);
+  [[maybe_unused]] uint2* h4 = reinterpret_cast<uint2*>(out_h + (WITH_H ? (size_t)row * width + base : 0));
 #pragma unroll
   for (int i = 0; i < 8; ++i)
-    if (base + 4 * i < width)
-      o4[i] = make_float4(r.q[i].x * inv * nw.q[i].x, r.q[i].y * inv * nw.q[i].y, r.q[i].z * inv * nw.q[i].z, r.q[i].w * inv * nw.q[i].w);
+    if (base + 4 * i < width) {
+      const float4 v = make_float4(r.q[i].x * inv * nw.q[i].x, r.q[i].y * inv * nw.q[i].y, r.q[i].z * inv * nw.q[i].z, r.q[i].w * inv * nw.q[i].w);
+      o4[i] = v;
+      if constexpr (WITH_H) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 lo = {(_Float16)v.x, (_Float16)v.y}, hi = {(_Float16)v.z, (_Float16)v.w};
+        h4[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+      }
+    }
 }
 
 __global__ void __launch_bounds__(256) k_route(const float* __restrict__ logits, const int* __restrict__ valid_tokens,
