@@ -259,7 +259,8 @@ int xabe_moe_block_set_fused_decode(xabe_moe_block* blk, int on);
 /* Measurement hook, no counterpart in the reference: ONE of the three decode launches (0: logits + shared
  * gate/up, 1: route + gate/up, 2: down + combine) with the arguments of xabe_moe_block_forward, so that a
  * launch can be timed and profiled alone.  Stage n reads what stages < n of an earlier call left in the
- * block's buffers; the live-token count is the one last published. */
+ * block's buffers; the live-token count is the one last published.  From eight tokens up stage 1 is two
+ * launches, the routing launch and the gate/up launch that reads its selections. */
 int xabe_moe_block_forward_stage(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w,
                                  const float* residual, size_t residual_len, const float* logit_bias, float* ffn_out,
                                  size_t ffn_out_len, float* l_out, size_t l_out_len, int stage);
