@@ -514,7 +514,7 @@ static int alloc_buffers(const xabe_moe_kernels* k, void* stream, int scope, boo
   A(&b->x_h, (wide && mma) ? g.max_tokens * g.hidden : 0);
   A(&b->inter_h, (wide && mma && routed) ? sorted * g.intermediate : 0);
   A(&b->shared_inter_h, (wide && mma) ? g.max_tokens * g.intermediate : 0);
-  b->n_tile_list = (wide && mma && routed) ? 4 * (eb + 1) + 4 : 0;
+  b->n_tile_list = (wide && mma && routed) ? 2 * (4 * (eb + 1) + 4) : 0;  // two lists (mfma_grouped_forward_partial)
   A(&b->tile_list, b->n_tile_list);
   b->n_router_partial = (mma && routed && g.max_tokens >= kRouterGemmMinTokens && router_gemm_splits(g) > 1)
                             ? (size_t)router_gemm_splits(g) * g.max_tokens * g.num_experts

@@ -10,7 +10,9 @@
 // gate rows and the matching 64 up rows, so SwiGLU happens in registers.  Token tiles come
 // from a device-built list with one entry per 128-slot chunk of every *active* expert's
 // run of the dispatch table: experts with no tokens cost nothing, whatever the skew.
-// Workgroups are persistent and stride over (token tile, row tile) items.
+// Workgroups are persistent and stride over (token tile, row tile) items.  (Token tiles are 64 rows while an
+// expert's share of a pass is small, and 384 rows on eight wavefronts for the routed gate/up launch of wide passes:
+// see k_mfma_expert's TBM.)
 //
 // Numerics.  Operands are fp16: activations rounded once; weights are (code - offset) exactly,
 // times fp16(d * sc * 256) -- the 2^8 keeps small scales out of the fp16 subnormal range and
@@ -175,14 +177,14 @@ __device__ __forceinline__ void q8_finish(const Q8Pend& p, Q8Raw& r) {
   r.dh = p.dh;
 }
 
-template <int QUANT>
+template <int QUANT, int UNITS>
 struct WRaw {
-  typename std::conditional<QUANT == kQ6K, Q6Pend, Q8Pend>::type u[2];
+  typename std::conditional<QUANT == kQ6K, Q6Pend, Q8Pend>::type u[UNITS];
 };
 
-// Global loads of one contraction step into registers: the raw blocks of this thread's two weight-row units.
-template <int QUANT>
-__device__ __forceinline__ void load_unit_w(int ks, int i, const uint8_t* const (&wrow)[2], int du, WRaw<QUANT>& wreg) {
+// Global loads of one contraction step into registers: the raw blocks of this thread's weight-row units.
+template <int QUANT, int UNITS>
+__device__ __forceinline__ void load_unit_w(int ks, int i, const uint8_t* const (&wrow)[UNITS], int du, WRaw<QUANT, UNITS>& wreg) {
   {
     if constexpr (QUANT == kQ6K) {
       // step ks covers half (ks & 1) of superblock ks >> 1
@@ -192,10 +194,10 @@ __device__ __forceinline__ void load_unit_w(int ks, int i, const uint8_t* const 
     }
   }
 }
-template <int QUANT>
-__device__ __forceinline__ void load_step_w(int ks, const uint8_t* const (&wrow)[2], int du, WRaw<QUANT>& wreg) {
-  load_unit_w<QUANT>(ks, 0, wrow, du, wreg);
-  load_unit_w<QUANT>(ks, 1, wrow, du, wreg);
+template <int QUANT, int UNITS>
+__device__ __forceinline__ void load_step_w(int ks, const uint8_t* const (&wrow)[UNITS], int du, WRaw<QUANT, UNITS>& wreg) {
+#pragma unroll
+  for (int i = 0; i < UNITS; ++i) load_unit_w<QUANT, UNITS>(ks, i, wrow, du, wreg);
 }
 
 #ifdef XABE_MFMA_TRACE
@@ -210,16 +212,29 @@ static __device__ long long g_mfma_trace[512 * 32 * 4];
 #define XABE_MT(slot) do { } while (0)
 #endif
 
-// TBM: token rows per tile, 128 or 64.  The narrow form serves geometries whose experts see at most ~64 tokens
+// TBM: token rows per tile, 384, 128 or 64.  The narrow form serves geometries whose experts see at most ~64 tokens
 // each (up to ~2000 tokens per pass): half the matrix instructions, activation bytes and output stores per
 // item, the same weight work.  A wavefront then owns 32 x 64 of the tile instead of 64 x 64; every output
-// element sees the same operands in the same order, so the two forms give the same bits.
+// element sees the same operands in the same order, so the forms give the same bits.
+// The tall form (384 token rows) is a workgroup of eight wavefronts, 4 x 2, each owning 96 x 64.  The vector
+// instructions of the dequantisation cost a SIMD more time than the matrix instructions they feed (39 % against 32 %
+// of the launch at 128 rows) and the two do not overlap, so what pays is dequantising a weight tile less often: at
+// ~256 rows per expert one tall tile holds all of an expert's rows, one dequantisation per expert and row tile
+// instead of two or three, one unit per thread and step instead of two.  A wavefront multiplies only the 32-row
+// blocks that hold live rows, and only live rows' activation pieces are requested.
 template <int QUANT, int NM, bool ROUTED, int TBM = 128>
-__global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
-  static_assert(TBM == 128 || TBM == 64, "token tile");
-  constexpr int MI = TBM / 64;       // 32-row blocks of the tile per wavefront
-  constexpr int kAPieces = TBM / 16; // 16-byte activation pieces per thread and step
-  // 67.5 KB of LDS per workgroup at 128 token rows (two per CU): dynamic, since the static limit is 64 KB
+__global__ void __launch_bounds__(TBM == 384 ? 512 : 256, 2) k_mfma_expert(MfmaArgs a) {
+  static_assert(TBM == 384 || TBM == 128 || TBM == 64, "token tile");
+  constexpr bool kTall = TBM == 384;
+  constexpr int kThreads = kTall ? 512 : 256;
+  constexpr int kUnits = 512 / kThreads;          // weight-row units (32 elements of a row) per thread and step
+  constexpr int MI = kTall ? 3 : TBM / 64;        // 32-row blocks of the tile per wavefront
+  // first tile row of block mi of wavefront row wm: consecutive blocks in the short forms; in the tall form block b of
+  // the tile belongs to wavefront row b % 4, so that the live rows (the first `rows` of the tile) spread evenly
+  constexpr int kBlockStride = kTall ? 128 : 32;  // rows between a wavefront's consecutive blocks
+  constexpr int kWaveStride = kTall ? 32 : 32 * MI;  // rows between consecutive wavefront rows' first blocks
+  constexpr int kAPieces = TBM * 16 / kThreads;   // 16-byte activation pieces per thread and step
+  // 67.5 KB of LDS per workgroup at 128 token rows (two per CU), 137 KB at 384: dynamic, since the static limit is 64 KB
   extern __shared__ __attribute__((aligned(16))) uint8_t mfma_smem[];
   _Float16* sA = reinterpret_cast<_Float16*>(mfma_smem);
   _Float16* sB = sA + TBM * kLdA;
@@ -229,7 +244,9 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   int* sOrow = sArow + TBM;                             // output row index, or -1 for a dead row
   float* sScale = reinterpret_cast<float*>(sOrow + TBM);
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // (tall form: uniform, so that the count of live blocks is a scalar and dead ones are branched around)
+  const int wave = kTall ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int valid = *a.valid_tokens;
   const int n_ntiles = a.n_rows / (NM == 2 ? 64 : 128);
@@ -299,11 +316,12 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     }
   };
   const ptrdiff_t up_minus_gate = NM == 2 ? a.w1 - a.w0 : 0;
-  const uint8_t* wrow[2];        // weight rows this thread dequantises
+  const uint8_t* wrow[kUnits];   // weight rows this thread dequantises
   uint32_t arow_off[kAPieces];   // activation chunks this thread moves, 16 bytes each per step: element offsets
+  [[maybe_unused]] uint32_t arow_live = ~0u;  // tall form: bit i set when piece i belongs to a live row
   auto set_wrow = [&](const Item& it) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < kUnits; ++i) {
       const int rb = rb0 + 64 * i;
       const uint8_t* base = a.w0;
       int wr;
@@ -319,13 +337,15 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       wrow[i] = base + (size_t)it.e * a.expert_bytes + (size_t)wr * row_bytes;
     }
   };
-  auto set_arow = [&](int buf) __attribute__((always_inline)) {
+  auto set_arow = [&](int buf, [[maybe_unused]] int live_rows) __attribute__((always_inline)) {
+    if constexpr (kTall) arow_live = 0u;
 #pragma unroll
     for (int i = 0; i < kAPieces; ++i) {
-      const int c = tid + 256 * i;
+      const int c = tid + kThreads * i;
       // piece c of the tile lands at LDS byte 16 c: row c >> 4, position c & 15, which holds chunk pos ^ (row & 15)
       const int row = c >> 4, chunk = (c & 15) ^ (row & 15);
       arow_off[i] = (uint32_t)sArow[buf * kTable + row] * (uint32_t)a.K + (uint32_t)chunk * 8u;
+      if constexpr (kTall) arow_live |= row < live_rows ? 1u << i : 0u;
     }
   };
 
@@ -339,8 +359,11 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   auto move_a = [&](int ks) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kAPieces; ++i) {
+      if constexpr (kTall) {
+        if (!(arow_live & (1u << i))) continue;  // (a dead row's slot in LDS keeps whatever it held: its products are dropped)
+      }
       const _Float16* src = a.a + ((size_t)arow_off[i] + (size_t)ks * kBK);
-      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_a + 4096u * i);  // + 16 * lane, by the hardware
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_a + (uint32_t)(kThreads * 16) * i);  // + 16 * lane, by the hardware
       // (m0 is named as clobbered so that the compiler sets it again before any use of its own; it warns that it
       // does not preserve the register across the statement, which is what is wanted here)
 #pragma clang diagnostic push
@@ -354,13 +377,14 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
   // activation tile (L2-warm) is moved during the step's own write phase, behind the dequantisation.  The contraction has an even
   // number of steps (whole superblocks), so the step pairs are unrolled and no register is copied.
   // (The down launch, NM = 1, has no registers to spare for the second step and keeps one in flight.)
-  constexpr int kWDepth = 2;
+  // (tall form: one step ahead; its steps are long enough, and a second set of raw registers does not fit)
+  constexpr int kWDepth = kTall ? 1 : 2;
   // load instructions one step's two units issue at the very least, one per separately addressed piece: Q6_K ql
   // low, ql high, qh, scales, d; Q8_0 the two 16-byte halves of the codes and d.  (No two pieces of a unit
   // are adjacent in memory except the scales and d, ten bytes that no single load covers, so the compiler cannot
   // issue fewer; issuing more only makes the barrier's wait stricter.)
-  constexpr int kWLoadsAtLeast = QUANT == kQ6K ? 10 : 6;
-  WRaw<QUANT> w[kWDepth];
+  constexpr int kWLoadsAtLeast = (QUANT == kQ6K ? 5 : 3) * kUnits;
+  WRaw<QUANT, kUnits> w[kWDepth];
 
   Item cur = decode(first);
   {
@@ -374,13 +398,13 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     }
     __syncthreads();
     set_wrow(cur);
-    set_arow(0);
+    set_arow(0, cur.rows);
     // (fenced apart: the waits the compiler places in the steps are the strictest any path into them needs, and
     // with these two sets of loads interleaved here it would make every step wait for its newest loads)
     order_fence();
-    load_step_w<QUANT>(0, wrow, du, w[0]);
+    load_step_w<QUANT, kUnits>(0, wrow, du, w[0]);
     order_fence();
-    if constexpr (kWDepth == 2) load_step_w<QUANT>(1, wrow, du, w[kWDepth - 1]);
+    if constexpr (kWDepth == 2) load_step_w<QUANT, kUnits>(1, wrow, du, w[kWDepth - 1]);
     order_fence();
   }
   int buf = 0;
@@ -428,7 +452,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       }
       move_a(ks);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < kUnits; ++i) {
         const int rb = rb0 + 64 * i;
         if constexpr (QUANT == kQ6K) {
           Q6Raw r;
@@ -456,7 +480,7 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       // path: the last two steps of a workgroup's last item re-read two of its own steps and drop them)
       const int ks_w = ks + kWDepth < nks ? ks + kWDepth : ks + kWDepth - nks;
       if (ks + kWDepth == nks && has_next) set_wrow(nxt);
-      load_step_w<QUANT>(ks_w, wrow, du, w[P]);
+      load_step_w<QUANT, kUnits>(ks_w, wrow, du, w[P]);
       XABE_MT(1);
       // Second barrier of the step, by hand: this wavefront's LDS stores and its activation pieces must have
       // landed, the weight loads just issued need not.  Memory operations retire in order, so "all but the last
@@ -466,36 +490,54 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
       asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kWLoadsAtLeast) : "memory");
       order_fence();
       XABE_MT(2);
-      if (ks + 1 == nks && has_next) set_arow(buf ^ 1);
-      const _Float16* pa = &sA[(wm * (TBM / 2) + (lane & 31)) * kLdA];
+      if (ks + 1 == nks && has_next) set_arow(buf ^ 1, nxt.rows);
+      const _Float16* pa = &sA[(wm * kWaveStride + (lane & 31)) * kLdA];
+      // 32-row blocks of this wavefront that hold live rows (all of them in the other forms)
+      const int nb = kTall ? min(max((cur.rows - wm * kWaveStride + kBlockStride - 1) / kBlockStride, 0), MI) : MI;
       const int swz = lane & 15, khalf = lane >> 5;  // (the row's low four bits are the lane's)
       const _Float16* pb = &sB[(wn * 64 + (lane & 31)) * kLd];
       const int wswz = w_swizzle(lane & 15);  // (the rows' low four bits are the lane's)
       // Operand fragments one sub-step ahead, in two register sets: the four LDS reads of sub-step kk + 1 are
       // issued before the four matrix instructions of sub-step kk, so their latency hides behind 128 cycles of
       // matrix work instead of standing between every group of four.
-      half8 fa[2][MI], fb[2][2];
-      auto frags = [&](int kk, int set) __attribute__((always_inline)) {
+      // (tall form: one register set for the activation fragments, read at the start of their sub-step: a second set
+      // does not fit beside 96 accumulators, and the SIMD's other wavefront multiplies while this one waits for LDS)
+      constexpr int kASets = kTall ? 1 : 2;
+      half8 fa[kASets][MI], fb[2][2];
+      auto frags_a = [&](int kk, int set) __attribute__((always_inline)) {
         const int apos = ((kk * 2 + khalf) ^ swz) * 8;
-        fa[set][0] = *reinterpret_cast<const half8*>(pa + apos);
-        if constexpr (MI == 2) fa[set][MI - 1] = *reinterpret_cast<const half8*>(pa + 32 * kLdA + apos);
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+          if (mi < nb) fa[set][mi] = *reinterpret_cast<const half8*>(pa + mi * kBlockStride * kLdA + apos);
+      };
+      auto frags_b = [&](int kk, int set) __attribute__((always_inline)) {
         const int bpos = ((kk * 2 + khalf) ^ wswz) * 8;
         fb[set][0] = *reinterpret_cast<const half8*>(pb + bpos);
         fb[set][1] = *reinterpret_cast<const half8*>(pb + 32 * kLd + bpos);
       };
-      frags(0, 0);
+      if (nb > 0) {
+        frags_a(0, 0);
+        frags_b(0, 0);
 #pragma unroll
-      for (int kk = 0; kk < kBK / 16; ++kk) {
-        const int c = kk & 1;
-        if (kk + 1 < kBK / 16) frags(kk + 1, c ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][0], fb[c][0], acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][0], fb[c][1], acc[0][1], 0, 0, 0);
-        if constexpr (MI == 2) {
-          acc[MI - 1][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][MI - 1], fb[c][0], acc[MI - 1][0], 0, 0, 0);
-          acc[MI - 1][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][MI - 1], fb[c][1], acc[MI - 1][1], 0, 0, 0);
+        for (int kk = 0; kk < kBK / 16; ++kk) {
+          const int c = kk & 1;
+          if (kk + 1 < kBK / 16) {
+            if constexpr (kASets == 2) frags_a(kk + 1, c ^ 1);
+            frags_b(kk + 1, c ^ 1);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int mi = 0; mi < MI; ++mi) {
+            if (mi < nb) {
+              acc[mi][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c % kASets][mi], fb[c][0], acc[mi][0], 0, 0, 0);
+              acc[mi][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c % kASets][mi], fb[c][1], acc[mi][1], 0, 0, 0);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (kASets == 1) {
+            if (kk + 1 < kBK / 16) frags_a(kk + 1, 0);
+          }
         }
-        __builtin_amdgcn_sched_barrier(0);
       }
       XABE_MT(3);
 #ifdef XABE_MFMA_TRACE
@@ -523,36 +565,49 @@ __global__ void __launch_bounds__(256, 2) k_mfma_expert(MfmaArgs a) {
     // token row: a quarter of the store instructions, but each touches 32 rows' cache lines with 32 bytes
     // instead of two rows' with 128, and the block took 1365 against 1333 us at 8192 tokens)
     // (the rows' table entries are all read first: one LDS round trip for the item instead of one per row)
-    int orows[MI][16];
-    [[maybe_unused]] float scs[MI][16];
+    // (tall form: one 32-row block at a time, skipping blocks without live rows: all three blocks' entries at once
+    // do not fit the registers beside 96 accumulators)
+    auto store_blocks = [&](auto first_c, auto count_c) __attribute__((always_inline)) {
+      constexpr int M0 = decltype(first_c)::value, MN = decltype(count_c)::value;
+      int orows[MN][16];
+      [[maybe_unused]] float scs[MN][16];
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
+      for (int mi = 0; mi < MN; ++mi) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int r = wm * (TBM / 2) + mi * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-        orows[mi][v] = sOrow[buf * kTable + r];
-        if (NM == 1) scs[mi][v] = sScale[buf * kTable + r];
+        for (int v = 0; v < 16; ++v) {
+          const int r = wm * kWaveStride + (M0 + mi) * kBlockStride + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+          orows[mi][v] = sOrow[buf * kTable + r];
+          if (NM == 1) scs[mi][v] = sScale[buf * kTable + r];
+        }
       }
-    }
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
+      for (int mi = 0; mi < MN; ++mi) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int orow = orows[mi][v];
-        if (orow < 0) continue;
-        if (NM == 2) {
-          const int col = cur.nt * 64 + wn * 32 + (lane & 31);
-          const float g = acc[mi][0][v] * kWScaleInv, u = acc[mi][1][v] * kWScaleInv;
-          static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_f(g) * u);
-        } else {
-          const float sc = scs[mi][v];
+        for (int v = 0; v < 16; ++v) {
+          const int orow = orows[mi][v];
+          if (orow < 0) continue;
+          if (NM == 2) {
+            const int col = cur.nt * 64 + wn * 32 + (lane & 31);
+            const float g = acc[M0 + mi][0][v] * kWScaleInv, u = acc[M0 + mi][1][v] * kWScaleInv;
+            static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_f(g) * u);
+          } else {
+            const float sc = scs[mi][v];
 #pragma unroll
-          for (int ni = 0; ni < 2; ++ni) {
-            const int col = cur.nt * 128 + wn * 64 + ni * 32 + (lane & 31);
-            static_cast<float*>(a.out)[(size_t)orow * a.n_rows + col] = sc * (acc[mi][ni][v] * kWScaleInv);
+            for (int ni = 0; ni < 2; ++ni) {
+              const int col = cur.nt * 128 + wn * 64 + ni * 32 + (lane & 31);
+              static_cast<float*>(a.out)[(size_t)orow * a.n_rows + col] = sc * (acc[M0 + mi][ni][v] * kWScaleInv);
+            }
           }
         }
       }
+    };
+    if constexpr (kTall) {
+      const int nb = min(max((cur.rows - wm * kWaveStride + kBlockStride - 1) / kBlockStride, 0), MI);
+      if (nb > 0) store_blocks(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+      if (nb > 1) store_blocks(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
+      if (nb > 2) store_blocks(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+    } else {
+      store_blocks(std::integral_constant<int, 0>{}, std::integral_constant<int, MI>{});
     }
     if (!has_next) break;
     cur = nxt;
@@ -645,6 +700,15 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
 static int routed_tile_rows(const xabe_moe_geometry& g) {
   return g.max_tokens * g.experts_per_token <= 48 * g.num_experts ? 64 : kBM;
 }
+// Token-tile height of the routed gate/up launch: the tall tile once an expert's share of a full pass fills most of it
+// (an average of 192 selections per expert: 6144 tokens of the model's shape).  Same-box, per block: 8192 tokens 1323
+// -> 1263 us (the launch itself 503 -> ~415), 6144 tokens 1081 -> 1043; at 4096 tokens (128 per expert) the tall tile
+// loses (778 against 767).  The down launch keeps the short tiles at every width: its contraction is four steps, its
+// items are mostly epilogue, and with tall tiles the block measured 1279 us against 1263.
+static int routed_up_tile_rows(const xabe_moe_geometry& g) {
+  if (g.max_tokens * g.experts_per_token >= 192 * g.num_experts) return 384;
+  return routed_tile_rows(g);
+}
 // The shared expert's launches are short of workgroups below a few thousand tokens: the narrow tile while all
 // of its items still start at once (two workgroups per compute unit), so that twice as many units share the work.
 static int shared_tile_rows(const xabe_moe_kernels* k, size_t row_tiles) {
@@ -676,6 +740,7 @@ int mfma_configure() {
   XABE_TRY((configure_one<2, false, 128>()));
   XABE_TRY((configure_one<2, true, 64>()));
   XABE_TRY((configure_one<2, true, 128>()));
+  XABE_TRY((configure_one<2, true, 384>()));
   done = true;
   return XABE_OK;
 }
@@ -683,11 +748,13 @@ int mfma_configure() {
 template <int NM, bool ROUTED, int TBM>
 static int launch_mfma(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
   // workgroups resident per CU: the narrow tile's registers (about 150) and LDS (49.5 KB) leave room for a third
-  const size_t per_cu = TBM == 64 ? 3 : 2;
+  // (the tall tile: eight wavefronts and 137 KB of LDS, one workgroup per CU)
+  const size_t per_cu = TBM == 64 ? 3 : TBM == 128 ? 2 : 1;
   const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus * per_cu));
   constexpr size_t smem = mfma_lds_bytes<TBM>();
-  if (quant == XABE_QUANT_Q6K) hipLaunchKernelGGL((k_mfma_expert<kQ6K, NM, ROUTED, TBM>), dim3(grid), dim3(256), smem, s, a);
-  else hipLaunchKernelGGL((k_mfma_expert<kQ8_0, NM, ROUTED, TBM>), dim3(grid), dim3(256), smem, s, a);
+  constexpr unsigned threads = TBM == 384 ? 512 : 256;
+  if (quant == XABE_QUANT_Q6K) hipLaunchKernelGGL((k_mfma_expert<kQ6K, NM, ROUTED, TBM>), dim3(grid), dim3(threads), smem, s, a);
+  else hipLaunchKernelGGL((k_mfma_expert<kQ8_0, NM, ROUTED, TBM>), dim3(grid), dim3(threads), smem, s, a);
   XABE_HIP_TRY(hipGetLastError());
   return XABE_OK;
 }
@@ -707,17 +774,24 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
                                  xabe_quant_tensor up, xabe_quant_tensor down, const float* x) {
   const xabe_moe_geometry& g = k->g;
   if (!b->x_h_ready) XABE_TRY(to_f16(k, s, b, x));
-  const int cap = (int)((b->n_tile_list - 4) / 4);
-  const int bm = routed_tile_rows(g);
+  // (the allocation holds two lists of the same capacity: the down launch's, and the gate/up launch's where its tile
+  // height differs)
+  const size_t list_ints = b->n_tile_list / 2;
+  const int cap = (int)((list_ints - 4) / 4);
+  const int bm = routed_tile_rows(g), bm_up = routed_up_tile_rows(g);
+  int* list_up = bm_up == bm ? b->tile_list : b->tile_list + list_ints;
   hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap, bm,
                      b->tile_list);
+  if (bm_up != bm)
+    hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap,
+                       bm_up, list_up);
   XABE_HIP_TRY(hipGetLastError());
   MfmaArgs a;
   memset(&a, 0, sizeof(a));
   a.valid_tokens = b->valid_tokens;
   a.sorted_token_ids = b->sorted_token_ids;
   a.topk_weights = b->topk_weights;
-  a.tile_list = b->tile_list;
+  a.tile_list = list_up;
   a.top_k = (int)g.experts_per_token;
   const size_t max_mtiles = (size_t)cap;
   // gate/up + SwiGLU -> inter_h[slot][I]
@@ -728,9 +802,11 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   a.out = b->inter_h;
   a.K = (int)g.hidden;
   a.n_rows = (int)g.intermediate;
-  if (bm == 64) XABE_TRY((launch_mfma<2, true, 64>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  if (bm_up == 64) XABE_TRY((launch_mfma<2, true, 64>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  else if (bm_up == 384) XABE_TRY((launch_mfma<2, true, 384>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
   else XABE_TRY((launch_mfma<2, true, 128>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
   // down -> partial[flat][H], scaled by the routing weight
+  a.tile_list = b->tile_list;
   a.w0 = static_cast<const uint8_t*>(down.bytes);
   a.w1 = nullptr;
   a.expert_bytes = g.hidden * stack_row_bytes(down.quant, g.intermediate);

@@ -171,6 +171,56 @@ def test_prefill_rows_do_not_depend_on_batch_mates(oracle, X):
     assert np.array_equal(la[5].view(np.uint32), lb[77].view(np.uint32))
 
 
+def test_tall_tiles_give_the_rows_of_the_short_tiles(oracle, X):
+    """From ~192 selections per expert up the routed gate/up launch runs 384-row token tiles (eight wavefronts, live
+    32-row blocks only); every output element still sees the same operands in the same order, so with the same
+    selections a token's routed row in an 8192-token pass is the bits it has in a 128-token pass, where the 64-row
+    tiles run."""
+    import torch
+
+    g_wide = X.MoeGeometry.qwen3_6(X.moe_block_size(8192), 8192)
+    g_small = X.MoeGeometry.qwen3_6(32, 128)
+    layer = make_layer(oracle, g_wide, seed=733)
+    d = layer.dev
+    rng = np.random.default_rng(9)
+    logits_s = rng.uniform(-3, 3, (128, 256)).astype(np.float32)
+    logits_w = rng.uniform(-3, 3, (8192, 256)).astype(np.float32)
+    xs = activations(36, 128, 2048)
+    xw = activations(37, 8192, 2048)
+    picks = [(0, 17), (5000, 5), (8191, 77), (4095, 127)]       # (row of the wide pass, row of the small pass)
+    for rw, r in picks:
+        xw[rw] = xs[r]
+        logits_w[rw] = logits_s[r]
+
+    def routed(g, tokens, logits, x):
+        k, b = _route_dispatch(X, g, tokens, logits)
+        assert k.tensor_cores_enabled()
+        out = torch.zeros(g.max_tokens, 2048, device="cuda")
+        k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)
+        torch.cuda.synchronize()
+        return out.cpu().numpy(), b.topk_ids().cpu().numpy()[:tokens * 8]
+
+    small, _ = routed(g_small, 128, logits_s, xs)
+    wide, ids = routed(g_wide, 8192, logits_w, xw)
+    # the wide pass did fill tall tiles: every expert took more than 128 rows and at most one tile's worth
+    counts = np.bincount(ids.ravel(), minlength=256)
+    assert counts.min() > 128 and counts.max() <= 384, (counts.min(), counts.max())
+    for rw, r in picks:
+        assert np.array_equal(wide[rw].view(np.uint32), small[r].view(np.uint32)), (rw, r)
+    # fewer live tokens in the same geometry: the experts' runs end inside the tall tiles' second blocks
+    wide2, ids2 = routed(g_wide, 6200, logits_w[:6200], xw)
+    assert np.bincount(ids2.ravel(), minlength=256).max() <= 256
+    for rw, r in picks[:2]:
+        assert np.array_equal(wide2[rw].view(np.uint32), small[r].view(np.uint32)), (rw, r)
+    assert np.all(wide2[6200:] == 0)
+    # and against the oracle, a few rows
+    k, b = _route_dispatch(X, g_wide, 8192, logits_w)
+    tw = b.topk_weights().cpu().numpy().reshape(8192, 8)
+    rows = [0, 5000, 8191]
+    ref = _naive(oracle, layer.host, xw.cpu().numpy()[rows], ids.reshape(8192, 8)[rows], tw[rows])
+    assert rel_to_peak(wide[rows], ref) <= MFMA_REL
+
+
 @pytest.mark.parametrize("router_q8", [True, False])
 def test_router_logits_matrix_core_path(oracle, X, router_q8):
     # from 2048 tokens up the router runs on the fp32 matrix instruction: fp32 operands, so the logits agree
