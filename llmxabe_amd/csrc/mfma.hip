@@ -629,49 +629,56 @@ __global__ void __launch_bounds__(256) k_to_f16_rows(const float* __restrict__ x
   }
 }
 
-// Token-tile list: one entry per `bm`-slot chunk of each active expert's run.  One workgroup.
+// Token-tile list: one entry per `bm`-slot chunk of each active expert's run.  One workgroup.  With bm_b > 0 a second
+// list of that tile height goes to tile_list_b in the same launch (the routed gate/up launch's, where it differs).
 __global__ void __launch_bounds__(256) k_build_tiles(const int* __restrict__ expert_counts, int num_experts, int block_size,
-                                                      int capacity, int bm, int* __restrict__ tile_list) {
+                                                      int capacity, int bm, int* __restrict__ tile_list, int bm_b,
+                                                      int* __restrict__ tile_list_b) {
   __shared__ int s_base[513], s_tiles[513];
   // exclusive prefixes of the padded run lengths and of the tile counts (num_experts <= 512): every thread
-  // takes two experts, the pair sums are scanned across the workgroup in nine doubling steps
+  // takes two experts, the pair sums are scanned across the workgroup in eight doubling steps
   __shared__ int s_scan[2][2][256];
   const int t = threadIdx.x;
-  int pad[2], til[2];
+  for (int pass = 0; pass < (bm_b > 0 ? 2 : 1); ++pass) {
+    const int h = pass ? bm_b : bm;
+    int* list = pass ? tile_list_b : tile_list;
+    int pad[2], til[2];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int e = 2 * t + j;
-    const int c = e < num_experts ? expert_counts[e] : 0;
-    pad[j] = (c + block_size - 1) / block_size * block_size;
-    til[j] = (c + bm - 1) / bm;
-  }
-  s_scan[0][0][t] = pad[0] + pad[1];
-  s_scan[0][1][t] = til[0] + til[1];
-  __syncthreads();
-  int cur = 0;
-  for (int d = 1; d < 256; d <<= 1) {
-#pragma unroll
-    for (int a = 0; a < 2; ++a) s_scan[cur ^ 1][a][t] = s_scan[cur][a][t] + (t >= d ? s_scan[cur][a][t - d] : 0);
-    cur ^= 1;
+    for (int j = 0; j < 2; ++j) {
+      const int e = 2 * t + j;
+      const int c = e < num_experts ? expert_counts[e] : 0;
+      pad[j] = (c + block_size - 1) / block_size * block_size;
+      til[j] = (c + h - 1) / h;
+    }
+    __syncthreads();  // (the previous pass has read its tables)
+    s_scan[0][0][t] = pad[0] + pad[1];
+    s_scan[0][1][t] = til[0] + til[1];
     __syncthreads();
-  }
-  {
-    const int base = s_scan[cur][0][t] - (pad[0] + pad[1]), tiles = s_scan[cur][1][t] - (til[0] + til[1]);
-    if (2 * t < num_experts) s_base[2 * t] = base, s_tiles[2 * t] = tiles;
-    if (2 * t + 1 < num_experts) s_base[2 * t + 1] = base + pad[0], s_tiles[2 * t + 1] = tiles + til[0];
-    if (t == 255) tile_list[0] = min(s_scan[cur][1][t], capacity);
-  }
-  __syncthreads();
-  for (int e = threadIdx.x; e < num_experts; e += 256) {
-    const int c = expert_counts[e];
-    const int nt = (c + bm - 1) / bm;
-    for (int i = 0; i < nt; ++i) {
-      const int idx = s_tiles[e] + i;
-      if (idx >= capacity) break;
-      tile_list[4 + 4 * idx + 0] = e;
-      tile_list[4 + 4 * idx + 1] = s_base[e] + i * bm;
-      tile_list[4 + 4 * idx + 2] = min(bm, c - i * bm);
-      tile_list[4 + 4 * idx + 3] = 0;
+    int cur = 0;
+    for (int d = 1; d < 256; d <<= 1) {
+#pragma unroll
+      for (int a = 0; a < 2; ++a) s_scan[cur ^ 1][a][t] = s_scan[cur][a][t] + (t >= d ? s_scan[cur][a][t - d] : 0);
+      cur ^= 1;
+      __syncthreads();
+    }
+    {
+      const int base = s_scan[cur][0][t] - (pad[0] + pad[1]), tiles = s_scan[cur][1][t] - (til[0] + til[1]);
+      if (2 * t < num_experts) s_base[2 * t] = base, s_tiles[2 * t] = tiles;
+      if (2 * t + 1 < num_experts) s_base[2 * t + 1] = base + pad[0], s_tiles[2 * t + 1] = tiles + til[0];
+      if (t == 255) list[0] = min(s_scan[cur][1][t], capacity);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < num_experts; e += 256) {
+      const int c = expert_counts[e];
+      const int nt = (c + h - 1) / h;
+      for (int i = 0; i < nt; ++i) {
+        const int idx = s_tiles[e] + i;
+        if (idx >= capacity) break;
+        list[4 + 4 * idx + 0] = e;
+        list[4 + 4 * idx + 1] = s_base[e] + i * h;
+        list[4 + 4 * idx + 2] = min(h, c - i * h);
+        list[4 + 4 * idx + 3] = 0;
+      }
     }
   }
 }
@@ -781,10 +788,7 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   const int bm = routed_tile_rows(g), bm_up = routed_up_tile_rows(g);
   int* list_up = bm_up == bm ? b->tile_list : b->tile_list + list_ints;
   hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap, bm,
-                     b->tile_list);
-  if (bm_up != bm)
-    hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap,
-                       bm_up, list_up);
+                     b->tile_list, bm_up != bm ? bm_up : 0, list_up);
   XABE_HIP_TRY(hipGetLastError());
   MfmaArgs a;
   memset(&a, 0, sizeof(a));
