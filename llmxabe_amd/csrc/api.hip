@@ -622,6 +622,13 @@ int xabe_moe_build_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_bu
     XABE_HIP_TRY(hipGetLastError());
     return XABE_OK;
   }
+  if (g.max_tokens * g.experts_per_token <= (size_t)kAlignFusedMaxSelections && g.num_experts <= 512) {
+    hipLaunchKernelGGL(k_align_fused, dim3(1), dim3(1024), 0, s, b->topk_ids, b->valid_tokens, (int)g.experts_per_token,
+                       (int)g.num_experts, (int)g.block_size, (int)b->n_sorted, (int)b->n_expert_blocks, b->sorted_token_ids,
+                       b->expert_ids, b->bucket_live, b->expert_counts, b->num_tokens_post_pad);
+    XABE_HIP_TRY(hipGetLastError());
+    return XABE_OK;
+  }
   hipLaunchKernelGGL(k_align_count, dim3((unsigned)g.num_experts), dim3(256), 0, s, b->topk_ids, b->valid_tokens,
                      (int)g.experts_per_token, (int)b->n_sorted, (int)b->n_expert_blocks, b->sorted_token_ids,
                      b->expert_ids, b->bucket_live, b->expert_counts);

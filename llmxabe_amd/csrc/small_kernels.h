@@ -239,6 +239,108 @@ __global__ void __launch_bounds__(256) k_align_scatter(const int* __restrict__ t
 }
 
 // ---------------------------------------------------------------------------------
+// The same tables from ONE launch of one workgroup, for passes of at most 8192 selections (1024 tokens of top-8):
+// the two launches above cost ~15 us at 512 tokens, nearly all of it launch and barrier latency (every expert's
+// workgroup walks all selections, two barriers per 256 of them).  Sixteen wavefronts split the selections into
+// sixteen consecutive ranges.  Each counts its range per expert (LDS atomics: only the totals are used), thread e
+// turns the sixteen counts of expert e into first slots (prefix over the ranges, plus the expert's base from a scan of
+// the padded totals), and each wavefront then ranks its selections among equals in index order, 64 at a time with
+// one ballot per bit of the id, and writes them.  No result depends on the order in which atomics land.
+// ---------------------------------------------------------------------------------
+constexpr int kAlignFusedMaxSelections = 8192;
+constexpr int kAlignFusedWaves = 16;
+__global__ void __launch_bounds__(1024) k_align_fused(const int* __restrict__ topk_ids, const int* __restrict__ valid_tokens,
+                                                       int top_k, int num_experts, int block_size, int sorted_capacity,
+                                                       int expert_capacity, int* __restrict__ sorted_token_ids,
+                                                       int* __restrict__ expert_ids, int* __restrict__ bucket_live,
+                                                       int* __restrict__ expert_counts, int* __restrict__ num_tokens_post_pad) {
+  constexpr int kMaxE = 512, kRounds = kAlignFusedMaxSelections / (kAlignFusedWaves * 64);
+  __shared__ int cnt[kAlignFusedWaves][kMaxE];  // per range and expert: count, then next slot
+  __shared__ int s_scan[2][kMaxE];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int numel = min(*valid_tokens * top_k, kAlignFusedMaxSelections);
+  // whole-capacity fill first: the barriers below order it before the entries written over it
+  for (int i = tid; i < sorted_capacity; i += 1024) sorted_token_ids[i] = numel;
+  for (int i = tid; i < expert_capacity; i += 1024) {
+    expert_ids[i] = -1;
+    bucket_live[i] = 0;
+  }
+  for (int i = tid; i < kAlignFusedWaves * kMaxE; i += 1024) (&cnt[0][0])[i] = 0;
+  __syncthreads();
+  const int per_range = ((numel + kAlignFusedWaves - 1) / kAlignFusedWaves + 63) / 64 * 64;
+  const int r0 = wave * per_range, r1 = min(r0 + per_range, numel);
+  int id[kRounds];
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const int i = r0 + r * 64 + lane;
+    id[r] = i < r1 ? topk_ids[i] : -1;
+    if (id[r] >= num_experts) id[r] = -1;  // (an id no expert has matches nothing, as in the two-launch form)
+    if (id[r] >= 0) atomicAdd(&cnt[wave][id[r]], 1);
+  }
+  __syncthreads();
+  int count = 0, padded = 0;
+  if (tid < kMaxE) {
+    if (tid < num_experts) {
+#pragma unroll
+      for (int w = 0; w < kAlignFusedWaves; ++w) {
+        const int h = cnt[w][tid];
+        cnt[w][tid] = count;  // selections of this expert in earlier ranges
+        count += h;
+      }
+      padded = (count + block_size - 1) / block_size * block_size;
+    }
+    s_scan[0][tid] = padded;
+  }
+  __syncthreads();
+  int cur = 0;
+  for (int d = 1; d < kMaxE; d <<= 1) {
+    if (tid < kMaxE) s_scan[cur ^ 1][tid] = s_scan[cur][tid] + (tid >= d ? s_scan[cur][tid - d] : 0);
+    cur ^= 1;
+    __syncthreads();
+  }
+  if (tid < kMaxE) {
+    const int base = s_scan[cur][tid] - padded;
+    if (tid == kMaxE - 1) *num_tokens_post_pad = s_scan[cur][tid];
+    if (tid < num_experts) {
+      expert_counts[tid] = count;
+#pragma unroll
+      for (int w = 0; w < kAlignFusedWaves; ++w) cnt[w][tid] += base;
+      const int nblk = (count + block_size - 1) / block_size;
+      for (int b = 0; b < nblk; ++b) {
+        const int blk = base / block_size + b;
+        if (blk < expert_capacity) {
+          expert_ids[blk] = tid;
+          bucket_live[blk] = min(block_size, count - b * block_size);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  int* mine = cnt[wave];
+  int id_bits = 1;
+  while ((1 << id_bits) < num_experts) ++id_bits;
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const int i = r0 + r * 64 + lane;
+    const int v = id[r];
+    unsigned long long same = __ballot(v >= 0);
+    for (int bit = 0; bit < id_bits; ++bit) {
+      const unsigned long long set = __ballot((v >> bit) & 1);
+      same &= ((v >> bit) & 1) ? set : ~set;
+    }
+    int pos = -1;
+    if (v >= 0) pos = mine[v] + __popcll(same & ((1ull << lane) - 1ull));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();  // every lane has read its expert's slot
+    if (v >= 0 && lane == __builtin_ctzll(same)) mine[v] += __popcll(same);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (pos >= 0 && pos < sorted_capacity) sorted_token_ids[pos] = i;
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // The same dispatch tables for prefill widths, as a stable counting sort in three launches whose work is
 // proportional to the number of selections (the two-launch form above has every expert's workgroup scan all
 // of them).  A chunk is 1024 consecutive flat ids, 256 per wavefront.
