@@ -64,6 +64,27 @@ def test_rms_norm_rows(oracle, X):
         X.LayerOpsKernels.rms_norm(x, w[:-1], out, rows, width, 1e-6)
 
 
+@pytest.mark.parametrize("rows,width", [(130, 2048), (64, 512), (67, 1000)])
+def test_rms_norm_short_rows_are_the_long_form_s_bits(oracle, X, rows, width):
+    """From 64 rows of at most 2048 elements one wavefront normalises a row, fetched and stored as consecutive
+    16-byte pieces through LDS; below that one workgroup does.  Both fold the row in the same order."""
+    import torch
+
+    x = X.synth_normal_f32(13, rows * width, 1.0).view(rows, width)
+    x[3] = 0
+    w = 1.0 + X.synth_normal_f32(14, width, 0.1)
+    out = torch.empty_like(x)
+    X.LayerOpsKernels.rms_norm(x, w, out, rows, width, 1e-6)
+    few = torch.empty(9, width, device="cuda")
+    X.LayerOpsKernels.rms_norm(x[:9].contiguous(), w, few, 9, width, 1e-6)
+    got, ref9 = out.cpu().numpy(), few.cpu().numpy()
+    assert np.array_equal(got[:9].view(np.uint32), ref9.view(np.uint32))
+    xn, wn = x.cpu().numpy(), w.cpu().numpy()
+    for r in (0, 3, rows - 1):
+        ref = oracle.rms_norm(xn[r], wn, 1e-6)
+        assert np.abs(got[r] - ref).max() <= 2e-6 * max(1.0, np.abs(ref).max()), r
+
+
 def _route(X, logits_np, max_tokens, tokens, E=256, K=8, block=32):
     import torch
 
@@ -151,7 +172,11 @@ def test_route_small_expert_counts(oracle, X):
 
 
 @pytest.mark.parametrize("tokens,max_tokens,block", [(37, 64, 32), (5, 8, 32), (200, 256, 32), (1500, 1536, 64),
-                                                     (8192, 8192, 64), (700, 8192, 64), (1025, 2048, 64)])
+                                                     (8192, 8192, 64), (700, 8192, 64), (1025, 2048, 64),
+                                                     # the one-launch form at and just under its 8192 selections
+                                                     (1024, 1024, 32), (1001, 1024, 32), (513, 1024, 64),
+                                                     # more chunks than the offsets kernel keeps in registers
+                                                     (12000, 16384, 64)])
 def test_dispatch_tables_are_exact(oracle, X, tokens, max_tokens, block):
     # moe_differential.rs:438-543: exact incl. padding, sentinel and -1 fill over the whole capacity
     r = oracle.Xorshift64Star(0xD15 + tokens)
