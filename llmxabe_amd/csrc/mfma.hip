@@ -704,22 +704,30 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
 // Token-tile height for a geometry: the narrow tile while an expert's share of a full pass usually fits in it
 // (an average of 48 selections per expert; at 64 every second expert overflows into a second tile, measured
 // 702 against 695 us at 2048 tokens).
-static int routed_tile_rows(const xabe_moe_geometry& g) {
-  return g.max_tokens * g.experts_per_token <= 48 * g.num_experts ? 64 : kBM;
+// `tokens`: pass_tokens() below.
+static int routed_tile_rows(const xabe_moe_geometry& g, size_t tokens) {
+  return tokens * g.experts_per_token <= 48 * g.num_experts ? 64 : kBM;
+}
+// The tokens a pass is known to hold when its launches are chosen: the live count last published to the device
+// scalar (a 512-token chunk run in buffers sized for 8192 should get the tiles of a 512-token pass), the buffers'
+// size before any was.  Every tile height serves any live count and gives the same bits, so a graph captured at one
+// count and replayed after another was published is slower at worst.
+static size_t pass_tokens(const xabe_moe_kernels* k, const xabe_moe_buffers* b) {
+  return b->valid_published > 0 ? std::min<size_t>((size_t)b->valid_published, k->g.max_tokens) : k->g.max_tokens;
 }
 // Token-tile height of the routed gate/up launch: the tall tile once an expert's share of a full pass fills most of it
 // (an average of 192 selections per expert: 6144 tokens of the model's shape).  Same-box, per block: 8192 tokens 1323
 // -> 1263 us (the launch itself 503 -> ~415), 6144 tokens 1081 -> 1043; at 4096 tokens (128 per expert) the tall tile
 // loses (778 against 767).  The down launch keeps the short tiles at every width: its contraction is four steps, its
 // items are mostly epilogue, and with tall tiles the block measured 1279 us against 1263.
-static int routed_up_tile_rows(const xabe_moe_geometry& g) {
-  if (g.max_tokens * g.experts_per_token >= 192 * g.num_experts) return 384;
-  return routed_tile_rows(g);
+static int routed_up_tile_rows(const xabe_moe_geometry& g, size_t tokens) {
+  if (tokens * g.experts_per_token >= 192 * g.num_experts) return 384;
+  return routed_tile_rows(g, tokens);
 }
 // The shared expert's launches are short of workgroups below a few thousand tokens: the narrow tile while all
 // of its items still start at once (two workgroups per compute unit), so that twice as many units share the work.
-static int shared_tile_rows(const xabe_moe_kernels* k, size_t row_tiles) {
-  return (k->g.max_tokens + 63) / 64 * row_tiles <= (size_t)k->num_cus * 2 ? 64 : kBM;
+static int shared_tile_rows(const xabe_moe_kernels* k, size_t tokens, size_t row_tiles) {
+  return (tokens + 63) / 64 * row_tiles <= (size_t)k->num_cus * 2 ? 64 : kBM;
 }
 
 // LDS a workgroup of the kernel asks for (dynamic: above the static limit).  The limit is raised per function,
@@ -785,7 +793,8 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   // height differs)
   const size_t list_ints = b->n_tile_list / 2;
   const int cap = (int)((list_ints - 4) / 4);
-  const int bm = routed_tile_rows(g), bm_up = routed_up_tile_rows(g);
+  const size_t tokens = pass_tokens(k, b);
+  const int bm = routed_tile_rows(g, tokens), bm_up = routed_up_tile_rows(g, tokens);
   int* list_up = bm_up == bm ? b->tile_list : b->tile_list + list_ints;
   hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap, bm,
                      b->tile_list, bm_up != bm ? bm_up : 0, list_up);
@@ -839,7 +848,7 @@ int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffer
   a.n_rows = (int)g.intermediate;
   {
     const size_t row_tiles = g.intermediate / 64;
-    const int bm = shared_tile_rows(k, row_tiles);
+    const int bm = shared_tile_rows(k, pass_tokens(k, b), row_tiles);
     const size_t items = (g.max_tokens + bm - 1) / bm * row_tiles;
     if (bm == 64) XABE_TRY((launch_mfma<2, false, 64>(k, gate.quant, a, items, s)));
     else XABE_TRY((launch_mfma<2, false, 128>(k, gate.quant, a, items, s)));
@@ -852,7 +861,7 @@ int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffer
   a.n_rows = (int)g.hidden;
   {
     const size_t row_tiles = g.hidden / 128;
-    const int bm = shared_tile_rows(k, row_tiles);
+    const int bm = shared_tile_rows(k, pass_tokens(k, b), row_tiles);
     const size_t items = (g.max_tokens + bm - 1) / bm * row_tiles;
     if (bm == 64) XABE_TRY((launch_mfma<1, false, 64>(k, down.quant, a, items, s)));
     else XABE_TRY((launch_mfma<1, false, 128>(k, down.quant, a, items, s)));
