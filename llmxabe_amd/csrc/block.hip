@@ -15,11 +15,23 @@ struct xabe_moe_block {
   float *normed, *logits, *routed, *shexp, *gate;
   size_t n_act, n_logits;
   int fused_decode;  // decode widths: the regrouped three-launch block where the shape allows
+  // matrix-core widths: the shared expert runs beside the router, the routing and the dispatch tables, on a stream
+  // of the block's own that forks from the caller's after the RMSNorm and joins it before the combine
+  hipStream_t side;
+  hipEvent_t forked, joined;
 };
 
 static int block_alloc(float** p, size_t n, hipStream_t s) {
   XABE_HIP_TRY(hipMalloc(reinterpret_cast<void**>(p), n * sizeof(float)));
   XABE_HIP_TRY(hipMemsetAsync(*p, 0, n * sizeof(float), s));
+  return XABE_OK;
+}
+
+// (default priority, like every stream this library makes)
+static int block_side_stream(xabe_moe_block* blk) {
+  XABE_HIP_TRY(hipStreamCreateWithFlags(&blk->side, hipStreamNonBlocking));
+  XABE_HIP_TRY(hipEventCreateWithFlags(&blk->forked, hipEventDisableTiming));
+  XABE_HIP_TRY(hipEventCreateWithFlags(&blk->joined, hipEventDisableTiming));
   return XABE_OK;
 }
 
@@ -40,6 +52,7 @@ int xabe_moe_block_new(const xabe_moe_geometry* geometry, float eps, void* strea
   if (st == XABE_OK) st = block_alloc(&blk->routed, blk->n_act, s);
   if (st == XABE_OK) st = block_alloc(&blk->shexp, blk->n_act, s);
   if (st == XABE_OK) st = block_alloc(&blk->gate, geometry->max_tokens, s);
+  if (st == XABE_OK && geometry->max_tokens >= kMfmaMinTokens) st = block_side_stream(blk);
   if (st != XABE_OK) {
     xabe_moe_block_free(blk);
     return st;
@@ -53,6 +66,9 @@ void xabe_moe_block_free(xabe_moe_block* blk) {
   float* ptrs[] = {blk->normed, blk->logits, blk->routed, blk->shexp, blk->gate};
   for (float* p : ptrs)
     if (p) (void)hipFree(p);
+  if (blk->forked) (void)hipEventDestroy(blk->forked);
+  if (blk->joined) (void)hipEventDestroy(blk->joined);
+  if (blk->side) (void)hipStreamDestroy(blk->side);
   xabe_moe_buffers_free(blk->buffers);
   xabe_moe_kernels_free(blk->moe);
   delete blk;
@@ -81,6 +97,22 @@ int xabe_moe_block_forward_stage(xabe_moe_block* blk, void* stream, const xabe_m
   XABE_TRY(check_layer_stacks(blk->moe, w));
   return launch_decode_block(blk->moe, as_stream(stream), blk->buffers, w, residual, logit_bias, blk->eps, blk->normed,
                              blk->logits, blk->shexp, blk->gate, blk->routed, ffn_out, l_out, 1u << stage);
+}
+
+// step 2 of the forward below: router logits, (bias,) softmax + top-k + renormalise, dispatch tables
+static int route_rows(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* logit_bias) {
+  const xabe_moe_geometry& g = blk->g;
+  if (!(w->router_quant < 0 || w->router_quant == XABE_QUANT_Q8_0))
+    return set_error(XABE_ERR_UNSUPPORTED_QUANT, "router: only f32 and Q8_0 routers are supported, got code %d", w->router_quant);
+  const size_t router_len = w->router_quant < 0
+                                ? g.num_experts * g.hidden
+                                : g.num_experts * g.hidden / xabe_expert_quant_block_elements(w->router_quant) *
+                                      xabe_expert_quant_block_bytes(w->router_quant);
+  bool bias_added = false;
+  XABE_TRY(router_logits_biased(blk->moe, stream, blk->buffers, w->router, router_len, w->router_quant, blk->normed,
+                                blk->n_act, blk->logits, blk->n_logits, logit_bias, &bias_added));
+  if (logit_bias && !bias_added) XABE_TRY(xabe_moe_add_logit_bias(blk->moe, stream, blk->buffers, logit_bias, blk->logits));
+  return xabe_moe_route_and_dispatch(blk->moe, stream, blk->buffers, blk->logits, blk->n_logits);
 }
 
 int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
@@ -112,44 +144,55 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
   if (!normed_h)
     XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
                            g.hidden, blk->eps));
-  // 2. router logits, (bias,) softmax + top-k + renormalise, dispatch tables
-  if (!(w->router_quant < 0 || w->router_quant == XABE_QUANT_Q8_0))
-    return set_error(XABE_ERR_UNSUPPORTED_QUANT, "router: only f32 and Q8_0 routers are supported, got code %d", w->router_quant);
-  const size_t router_len = w->router_quant < 0
-                                ? g.num_experts * g.hidden
-                                : g.num_experts * g.hidden / xabe_expert_quant_block_elements(w->router_quant) *
-                                      xabe_expert_quant_block_bytes(w->router_quant);
-  bool bias_added = false;
-  XABE_TRY(router_logits_biased(blk->moe, stream, blk->buffers, w->router, router_len, w->router_quant, blk->normed,
-                                blk->n_act, blk->logits, blk->n_logits, logit_bias, &bias_added));
-  if (logit_bias && !bias_added) XABE_TRY(xabe_moe_add_logit_bias(blk->moe, stream, blk->buffers, logit_bias, blk->logits));
-  XABE_TRY(xabe_moe_route_and_dispatch(blk->moe, stream, blk->buffers, blk->logits, blk->n_logits));
-  // 3 + 4. routed experts (stopping at `partial`) and the ungated shared expert
-  int fused = 0;
-  if (!wide)
-    XABE_TRY(xabe_moe_grouped_forward_partial_with_shared(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps,
-                                                          w->down_exps, w->shared_gate, w->shared_up, w->shared_down,
-                                                          blk->normed, blk->n_act, blk->shexp, blk->n_act, &fused));
-  if (!fused) {
-    const bool shared_mma =
-        wide && mfma_supported(blk->moe, blk->buffers, w->shared_gate.quant, w->shared_up.quant, w->shared_down.quant, false);
-    // the routed and the shared matrix-core paths read the same fp16 copy of the rows: made once here
-    if (normed_h) {
-      blk->buffers->x_h_ready = true;
-    } else if (shared_mma) {
-      XABE_TRY(mfma_convert_activations(blk->moe, as_stream(stream), blk->buffers, blk->normed));
-      blk->buffers->x_h_ready = true;
-    }
-    int st = xabe_moe_grouped_forward_partial(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps, w->down_exps,
-                                              blk->normed, blk->n_act);
-    if (st == XABE_OK && shared_mma)
-      st = xabe_moe_shared_expert_mma(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
-                                      blk->normed, blk->n_act, blk->shexp, blk->n_act);
-    else if (st == XABE_OK)
-      st = xabe_moe_shared_expert(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
-                                  blk->normed, blk->n_act, blk->shexp, blk->n_act);
+  const bool shared_mma =
+      wide && mfma_supported(blk->moe, blk->buffers, w->shared_gate.quant, w->shared_up.quant, w->shared_down.quant, false);
+  if (shared_mma && blk->side) {
+    // Matrix-core widths: the shared expert needs the rows only, so it forks off here and runs beside steps 2 and 3,
+    // whose first launches (router, routing, dispatch tables, tile lists) leave most of the device idle.
+    hipStream_t s = as_stream(stream);
+    if (!normed_h) XABE_TRY(mfma_convert_activations(blk->moe, s, blk->buffers, blk->normed));
+    XABE_HIP_TRY(hipEventRecord(blk->forked, s));
+    XABE_HIP_TRY(hipStreamWaitEvent(blk->side, blk->forked, 0));
+    blk->buffers->x_h_ready = true;  // both expert paths read the fp16 copy of the rows made above
+    int st = xabe_moe_shared_expert_mma(blk->moe, blk->side, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
+                                        blk->normed, blk->n_act, blk->shexp, blk->n_act);
+    hipError_t he = hipEventRecord(blk->joined, blk->side);
+    if (st == XABE_OK) st = route_rows(blk, stream, w, logit_bias);
+    if (st == XABE_OK)
+      st = xabe_moe_grouped_forward_partial(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps, w->down_exps, blk->normed,
+                                            blk->n_act);
     blk->buffers->x_h_ready = false;
+    // (whatever happened above, the caller's stream takes the side stream back)
+    if (he == hipSuccess) he = hipStreamWaitEvent(s, blk->joined, 0);
     if (st != XABE_OK) return st;
+    XABE_HIP_TRY(he);
+  } else {
+    XABE_TRY(route_rows(blk, stream, w, logit_bias));
+    // 3 + 4. routed experts (stopping at `partial`) and the ungated shared expert
+    int fused = 0;
+    if (!wide)
+      XABE_TRY(xabe_moe_grouped_forward_partial_with_shared(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps,
+                                                            w->down_exps, w->shared_gate, w->shared_up, w->shared_down,
+                                                            blk->normed, blk->n_act, blk->shexp, blk->n_act, &fused));
+    if (!fused) {
+      // the routed and the shared matrix-core paths read the same fp16 copy of the rows: made once here
+      if (normed_h) {
+        blk->buffers->x_h_ready = true;
+      } else if (shared_mma) {
+        XABE_TRY(mfma_convert_activations(blk->moe, as_stream(stream), blk->buffers, blk->normed));
+        blk->buffers->x_h_ready = true;
+      }
+      int st = xabe_moe_grouped_forward_partial(blk->moe, stream, blk->buffers, w->gate_exps, w->up_exps, w->down_exps,
+                                                blk->normed, blk->n_act);
+      if (st == XABE_OK && shared_mma)
+        st = xabe_moe_shared_expert_mma(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
+                                        blk->normed, blk->n_act, blk->shexp, blk->n_act);
+      else if (st == XABE_OK)
+        st = xabe_moe_shared_expert(blk->moe, stream, blk->buffers, w->shared_gate, w->shared_up, w->shared_down,
+                                    blk->normed, blk->n_act, blk->shexp, blk->n_act);
+      blk->buffers->x_h_ready = false;
+      if (st != XABE_OK) return st;
+    }
   }
   // 5. routed sum, sigmoid gate, combine, residual
   return xabe_moe_gate_and_combine(blk->moe, stream, blk->buffers, w->shared_gate_inp, blk->normed, blk->shexp, residual,

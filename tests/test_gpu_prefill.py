@@ -221,6 +221,49 @@ def test_tall_tiles_give_the_rows_of_the_short_tiles(oracle, X):
     assert rel_to_peak(wide[rows], ref) <= MFMA_REL
 
 
+def test_wide_block_passes_back_to_back_keep_their_own_shared_rows(oracle, X):
+    """At matrix-core widths the shared expert runs on a stream of the block's own, forked from the caller's after the
+    RMSNorm and joined before the combine.  Passes issued back to back on one block, alternating two inputs, must each
+    give the bits of the same pass run alone: a pass's shared rows are not read before they are written, nor
+    overwritten by the next pass before its combine has read them.  Eagerly on a caller's stream, and as a captured
+    graph replayed with eager passes between the replays."""
+    import torch
+
+    tokens = 512
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(tokens), tokens)
+    layer = make_layer(oracle, g, seed=710)
+    xa, xb = activations(41, tokens, 2048), activations(42, tokens, 2048)
+    blk = X.MoeBlock(g)
+    alone = {}
+    for name, x in (("a", xa), ("b", xb)):
+        ffn, lout = run_block(blk, layer, x, tokens)
+        torch.cuda.synchronize()
+        alone[name] = (ffn.view(torch.int32).clone(), blk.shared_ungated().view(torch.int32).clone())
+    assert not torch.equal(alone["a"][0], alone["b"][0])
+    stream = torch.cuda.Stream()
+    outs = [(torch.zeros_like(xa), torch.zeros_like(xa)) for _ in range(8)]
+    with torch.cuda.stream(stream):
+        for i, (ffn, lout) in enumerate(outs):
+            blk.forward(layer.dev, xa if i % 2 == 0 else xb, tokens, ffn, lout)
+        stream.synchronize()
+        for i, (ffn, _) in enumerate(outs):
+            assert torch.equal(ffn.view(torch.int32), alone["ab"[i % 2]][0]), f"pass {i} of 8 back to back"
+        # captured: two passes in one graph (a then b), replayed with an eager pass of the other input in between
+        (fa, la), (fb, lb) = outs[0], outs[1]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            blk.forward(layer.dev, xa, tokens, fa, la)
+            blk.forward(layer.dev, xb, tokens, fb, lb)
+        for rep in range(3):
+            fa.fill_(float("nan")); fb.fill_(float("nan"))
+            blk.forward(layer.dev, xb if rep % 2 == 0 else xa, tokens, outs[2][0], outs[2][1])
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(fa.view(torch.int32), alone["a"][0]), f"replay {rep}, first pass"
+            assert torch.equal(fb.view(torch.int32), alone["b"][0]), f"replay {rep}, second pass"
+            assert torch.equal(blk.shared_ungated().view(torch.int32), alone["b"][1]), f"replay {rep}, shared rows"
+
+
 @pytest.mark.parametrize("router_q8", [True, False])
 def test_router_logits_matrix_core_path(oracle, X, router_q8):
     # from 2048 tokens up the router runs on the fp32 matrix instruction: fp32 operands, so the logits agree
