@@ -245,7 +245,10 @@ int xabe_moe_block_new(const xabe_moe_geometry* geometry, float eps, void* strea
 void xabe_moe_block_free(xabe_moe_block* blk);
 int xabe_moe_block_publish_tokens(xabe_moe_block* blk, void* stream, size_t tokens); /* B:1081-1089 */
 /* MoeBlock::forward (B:1091-1329).  residual / ffn_out / l_out are [max_tokens][hidden];
- * `logit_bias` (may be NULL) is added to the router logits before routing. */
+ * `logit_bias` (may be NULL) is added to the router logits before routing.
+ * From 64 tokens up the shared expert's launches go to a stream the handle owns, forked from `stream` after the
+ * RMSNorm and joined to it before the combine (event record / wait only, capturable): work the caller enqueues on
+ * `stream` after the call is ordered after all of it.  One handle serves one stream at a time. */
 int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
                            size_t residual_len, size_t tokens, const float* logit_bias, float* ffn_out,
                            size_t ffn_out_len, float* l_out, size_t l_out_len);
