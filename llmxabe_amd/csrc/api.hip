@@ -609,6 +609,21 @@ int xabe_moe_build_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_bu
   XABE_TRY(require_routed(b, "build_dispatch"));
   const xabe_moe_geometry& g = k->g;
   hipStream_t s = as_stream(stream);
+  // the matrix-core grouped GEMM's token-tile lists come out of the same launch where one workgroup holds every
+  // expert's count and first slot; the heights they were cut for are noted for the launch that reads them
+  TileListArgs tl;
+  memset(&tl, 0, sizeof(tl));
+  b->tiles_bm = b->tiles_bm_up = 0;
+  XABE_TRY(stream_capture_id(s, &b->tiles_capture));
+  int bm = 0, bm_up = 0, cap = 0;
+  const bool lists = mfma_tile_plan(k, b, &bm, &bm_up, &cap) && g.num_experts <= 512;
+  if (lists) {
+    tl.capacity = cap;
+    tl.bm = bm;
+    tl.list = b->tile_list;
+    tl.bm_b = bm_up != bm ? bm_up : 0;
+    tl.list_b = b->tile_list + b->n_tile_list / 2;
+  }
   if (b->n_align_chunks) {
     const unsigned chunks = (unsigned)b->n_align_chunks;
     hipLaunchKernelGGL(k_align_hist, dim3(chunks), dim3(256), 0, s, b->topk_ids, b->valid_tokens, (int)g.experts_per_token,
@@ -616,17 +631,19 @@ int xabe_moe_build_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_bu
                        b->expert_ids, b->bucket_live);
     hipLaunchKernelGGL(k_align_offsets, dim3(1), dim3(512), 0, s, b->valid_tokens, (int)g.experts_per_token,
                        (int)g.num_experts, (int)g.block_size, (int)chunks, (int)b->n_expert_blocks, b->align_hist,
-                       b->expert_counts, b->expert_ids, b->bucket_live, b->num_tokens_post_pad);
+                       b->expert_counts, b->expert_ids, b->bucket_live, b->num_tokens_post_pad, tl);
     hipLaunchKernelGGL(k_align_place, dim3(chunks), dim3(256), 0, s, b->topk_ids, b->valid_tokens, (int)g.experts_per_token,
                        (int)g.num_experts, (int)b->n_sorted, b->align_hist, b->sorted_token_ids);
     XABE_HIP_TRY(hipGetLastError());
+    if (lists) b->tiles_bm = bm, b->tiles_bm_up = bm_up;
     return XABE_OK;
   }
   if (g.max_tokens * g.experts_per_token <= (size_t)kAlignFusedMaxSelections && g.num_experts <= 512) {
     hipLaunchKernelGGL(k_align_fused, dim3(1), dim3(1024), 0, s, b->topk_ids, b->valid_tokens, (int)g.experts_per_token,
                        (int)g.num_experts, (int)g.block_size, (int)b->n_sorted, (int)b->n_expert_blocks, b->sorted_token_ids,
-                       b->expert_ids, b->bucket_live, b->expert_counts, b->num_tokens_post_pad);
+                       b->expert_ids, b->bucket_live, b->expert_counts, b->num_tokens_post_pad, tl);
     XABE_HIP_TRY(hipGetLastError());
+    if (lists) b->tiles_bm = bm, b->tiles_bm_up = bm_up;
     return XABE_OK;
   }
   hipLaunchKernelGGL(k_align_count, dim3((unsigned)g.num_experts), dim3(256), 0, s, b->topk_ids, b->valid_tokens,
@@ -647,6 +664,28 @@ int xabe_moe_route_and_dispatch(const xabe_moe_kernels* k, void* stream, xabe_mo
   XABE_TRY(require_routed(b, "route_and_dispatch"));
   XABE_TRY(xabe_moe_route(k, stream, b, logits, logits_len));
   if (flat_regime(k)) return XABE_OK;  // the flat kernels read topk_ids directly
+  return xabe_moe_build_dispatch(k, stream, b);
+}
+
+int xabe::route_planes_and_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, float* logits,
+                                    size_t logits_len, const float* bias) {
+  if (!k || !b || !logits) return set_error(XABE_ERR_INVALID_ARGUMENT, "route: null pointer");
+  XABE_TRY(require_routed(b, "route"));
+  const xabe_moe_geometry& g = k->g;
+  if (g.num_experts > kRouteMaxExperts)
+    return bad_geometry(g, "the routing wavefront holds 8 experts per lane, so at most 512 experts");
+  if (g.experts_per_token > 64) return bad_geometry(g, "the routing wavefront keeps one selection per lane, so at most top-64");
+  XABE_TRY(check_len("logits", g.max_tokens * g.num_experts, logits_len));
+  const int splits = router_gemm_splits(g);
+  if (!b->router_partial || splits < 2 || splits > 8 || b->n_router_partial < (size_t)splits * g.max_tokens * g.num_experts)
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "route: no partial logit planes to route from");
+  const unsigned grid = (unsigned)((g.max_tokens + 3) / 4);
+  const size_t smem = 4 * g.num_experts * sizeof(float);
+  hipLaunchKernelGGL(k_route_planes, dim3(grid), dim3(256), smem, as_stream(stream), b->router_partial,
+                     g.max_tokens * g.num_experts, splits, bias, b->valid_tokens, (int)g.num_experts, (int)g.experts_per_token,
+                     logits, b->topk_ids, b->topk_weights);
+  XABE_HIP_TRY(hipGetLastError());
+  if (flat_regime(k)) return XABE_OK;
   return xabe_moe_build_dispatch(k, stream, b);
 }
 
@@ -950,8 +989,9 @@ int xabe_moe_router_logits(const xabe_moe_kernels* k, void* stream, const xabe_m
 
 int xabe::router_logits_biased(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b, const void* router,
                                size_t router_len, int router_quant, const float* normed, size_t normed_len, float* logits,
-                               size_t logits_len, const float* bias, bool* bias_added) {
+                               size_t logits_len, const float* bias, bool* bias_added, bool* sum_deferred) {
   if (bias_added) *bias_added = false;
+  if (sum_deferred) *sum_deferred = false;
   if (!k || !b || !router || !normed || !logits) return set_error(XABE_ERR_INVALID_ARGUMENT, "router_logits: null pointer");
   const xabe_moe_geometry& g = k->g;
   const size_t elems = g.num_experts * g.hidden;
@@ -970,7 +1010,7 @@ int xabe::router_logits_biased(const xabe_moe_kernels* k, void* stream, const xa
   XABE_TRY(check_len("normed", g.max_tokens * g.hidden, normed_len));
   XABE_TRY(check_len("logits", g.max_tokens * g.num_experts, logits_len));
   if (router_gemm_supported(k, b, fmt))
-    return launch_router_gemm(k, as_stream(stream), b, router, fmt, normed, logits, bias, bias_added);
+    return launch_router_gemm(k, as_stream(stream), b, router, fmt, normed, logits, bias, bias_added, sum_deferred);
   ExpertArgs a = base_args(k, b);
   a.w0 = static_cast<const uint8_t*>(router);
   a.x = normed;

@@ -108,9 +108,11 @@ static int route_rows(xabe_moe_block* blk, void* stream, const xabe_moe_layer_we
                                 ? g.num_experts * g.hidden
                                 : g.num_experts * g.hidden / xabe_expert_quant_block_elements(w->router_quant) *
                                       xabe_expert_quant_block_bytes(w->router_quant);
-  bool bias_added = false;
+  bool bias_added = false, planes = false;
   XABE_TRY(router_logits_biased(blk->moe, stream, blk->buffers, w->router, router_len, w->router_quant, blk->normed,
-                                blk->n_act, blk->logits, blk->n_logits, logit_bias, &bias_added));
+                                blk->n_act, blk->logits, blk->n_logits, logit_bias, &bias_added, &planes));
+  // (a split router GEMM leaves partial planes: the routing launch adds them, and the bias, as it reads them)
+  if (planes) return route_planes_and_dispatch(blk->moe, stream, blk->buffers, blk->logits, blk->n_logits, logit_bias);
   if (logit_bias && !bias_added) XABE_TRY(xabe_moe_add_logit_bias(blk->moe, stream, blk->buffers, logit_bias, blk->logits));
   return xabe_moe_route_and_dispatch(blk->moe, stream, blk->buffers, blk->logits, blk->n_logits);
 }

@@ -40,6 +40,14 @@ int validate_geometry(const xabe_moe_geometry& g);  // MoeKernels::new's checks 
   } while (0)
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+// id of the capture `s` is recording into, 0 when it is not capturing
+inline int stream_capture_id(hipStream_t s, unsigned long long* id) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long cid = 0;
+  XABE_HIP_TRY(hipStreamGetCaptureInfo(s, &status, &cid));
+  *id = status == hipStreamCaptureStatusActive ? cid : 0;
+  return XABE_OK;
+}
 
 }  // namespace xabe
 
@@ -84,12 +92,17 @@ inline int router_gemm_splits(const xabe_moe_geometry& g) {
 bool router_gemm_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int router_quant);
 int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,
                        int router_quant, const float* normed, float* logits, const float* bias = nullptr,
-                       bool* bias_added = nullptr);
+                       bool* bias_added = nullptr, bool* sum_deferred = nullptr);
 // Router logits with the per-expert bias folded into the launch that finishes them where there is one (the split
 // matrix-instruction GEMM's plane sum); `*bias_added` says whether it was (otherwise the caller adds it).
+// `sum_deferred` (may be null): where the logits come out as the partial planes of a split contraction, leave them
+// so and say so in *sum_deferred; the caller then routes with route_planes_and_dispatch, which adds the planes (and
+// the bias) in the same order in the routing launch and writes `logits` there.
 int router_logits_biased(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b, const void* router,
                          size_t router_len, int router_quant, const float* normed, size_t normed_len, float* logits,
-                         size_t logits_len, const float* bias, bool* bias_added);
+                         size_t logits_len, const float* bias, bool* bias_added, bool* sum_deferred = nullptr);
+int route_planes_and_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_buffers* b, float* logits, size_t logits_len,
+                              const float* bias);
 // RMSNorm of `rows` rows that also writes the fp16 copy the matrix-core kernels read (rows of at most 2048
 // elements, at least 64 of them); returns false in *done when the shape is not served.
 int rms_norm_rows_with_f16(void* stream, const float* x, const float* weight, float* out, void* out_h, size_t rows,
@@ -98,6 +111,9 @@ int rms_norm_rows_with_f16(void* stream, const float* x, const float* weight, fl
 int mfma_configure();
 int long_rows_configure();
 bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int gate_q, int up_q, int down_q, bool routed);
+// token-tile heights of the routed down and gate/up launches of the pass as published, and the entries one of the two
+// lists in `tile_list` holds; false when these buffers carry no lists
+bool mfma_tile_plan(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int* bm, int* bm_up, int* capacity);
 int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
                                  xabe_quant_tensor up, xabe_quant_tensor down, const float* x);
 int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, xabe_quant_tensor gate,
@@ -145,6 +161,11 @@ struct xabe_moe_buffers {
   uint16_t* shared_inter_h;
   int32_t* tile_list;   // device-built tile schedule
   size_t n_tile_list;
+  // tile heights the lists were cut for by the last dispatch build (0: not built there), and the capture that
+  // build was recorded into (0: launched eagerly): a forward trusts the lists only inside the same capture, or
+  // eagerly after an eager build, so that a captured forward never depends on lists made outside its graph
+  int tiles_bm, tiles_bm_up;
+  unsigned long long tiles_capture;
   float* router_partial;  // [split][token][expert]: the router GEMM's contraction splits at mid widths
   size_t n_router_partial;
   size_t bytes;

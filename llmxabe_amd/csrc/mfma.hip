@@ -730,6 +730,15 @@ static int shared_tile_rows(const xabe_moe_kernels* k, size_t tokens, size_t row
   return (tokens + 63) / 64 * row_tiles <= (size_t)k->num_cus * 2 ? 64 : kBM;
 }
 
+bool mfma_tile_plan(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int* bm, int* bm_up, int* capacity) {
+  if (!b->tile_list || b->n_tile_list < 16 || !k->tensor_cores || k->exact_regime) return false;
+  const size_t tokens = pass_tokens(k, b);
+  *bm = routed_tile_rows(k->g, tokens);
+  *bm_up = routed_up_tile_rows(k->g, tokens);
+  *capacity = (int)((b->n_tile_list / 2 - 4) / 4);
+  return true;
+}
+
 // LDS a workgroup of the kernel asks for (dynamic: above the static limit).  The limit is raised per function,
 // once, when a kernels handle is created (mfma_configure): nothing on the launch path but the launch.
 template <int TBM>
@@ -792,13 +801,17 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   // (the allocation holds two lists of the same capacity: the down launch's, and the gate/up launch's where its tile
   // height differs)
   const size_t list_ints = b->n_tile_list / 2;
-  const int cap = (int)((list_ints - 4) / 4);
-  const size_t tokens = pass_tokens(k, b);
-  const int bm = routed_tile_rows(g, tokens), bm_up = routed_up_tile_rows(g, tokens);
+  int bm, bm_up, cap;
+  (void)mfma_tile_plan(k, b, &bm, &bm_up, &cap);
   int* list_up = bm_up == bm ? b->tile_list : b->tile_list + list_ints;
-  hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap, bm,
-                     b->tile_list, bm_up != bm ? bm_up : 0, list_up);
-  XABE_HIP_TRY(hipGetLastError());
+  // (the dispatch build has usually left the lists, cut for these heights)
+  unsigned long long capture = 0;
+  XABE_TRY(stream_capture_id(s, &capture));
+  if (b->tiles_bm != bm || b->tiles_bm_up != bm_up || b->tiles_capture != capture) {
+    hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap,
+                       bm, b->tile_list, bm_up != bm ? bm_up : 0, list_up);
+    XABE_HIP_TRY(hipGetLastError());
+  }
   MfmaArgs a;
   memset(&a, 0, sizeof(a));
   a.valid_tokens = b->valid_tokens;

@@ -145,8 +145,10 @@ bool router_gemm_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b,
 }
 
 int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_buffers* b, const void* router,
-                       int router_quant, const float* normed, float* logits, const float* bias, bool* bias_added) {
+                       int router_quant, const float* normed, float* logits, const float* bias, bool* bias_added,
+                       bool* sum_deferred) {
   if (bias_added) *bias_added = false;
+  if (sum_deferred) *sum_deferred = false;
   const xabe_moe_geometry& g = k->g;
   RouterGemmArgs a;
   memset(&a, 0, sizeof(a));
@@ -162,7 +164,9 @@ int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_
   if (router_quant < 0) hipLaunchKernelGGL(k_router_gemm<false>, grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL(k_router_gemm<true>, grid, dim3(256), 0, s, a);
   XABE_HIP_TRY(hipGetLastError());
-  if (a.splits > 1) {
+  if (a.splits > 1 && sum_deferred) {
+    *sum_deferred = true;  // the caller's routing launch adds the planes (k_route_planes)
+  } else if (a.splits > 1) {
     const size_t n = g.max_tokens * g.num_experts;
     hipLaunchKernelGGL(k_router_sum_planes, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, b->router_partial,
                        b->valid_tokens, a.splits, a.max_tokens, a.E, bias, logits);

@@ -145,6 +145,35 @@ __global__ void __launch_bounds__(256) k_route(const float* __restrict__ logits,
   }
 }
 
+// The same routing for logits that a split router GEMM left as partial planes: a token's wavefront adds its row of
+// the planes (and the bias) in the order of k_router_sum_planes, writes the finished logits, and routes them.
+__global__ void __launch_bounds__(256) k_route_planes(const float* __restrict__ planes, size_t plane_stride, int splits,
+                                                       const float* __restrict__ bias, const int* __restrict__ valid_tokens,
+                                                       int num_experts, int top_k, float* __restrict__ logits,
+                                                       int* __restrict__ topk_ids, float* __restrict__ topk_weights) {
+  extern __shared__ float route_smem[];  // 4 x num_experts
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= *valid_tokens) return;
+  int sel_i;
+  float sel_w;
+  const size_t row = (size_t)t * num_experts;
+  float* e_all = route_smem + (size_t)wave * num_experts;
+  if (num_experts <= 256) {
+    float l[4];
+    route_load_planes<4>(planes + row, plane_stride, splits, num_experts, bias, logits + row, l);
+    route_compute<4>(l, num_experts, top_k, e_all, sel_i, sel_w);
+  } else {
+    float l[kRouteMaxPerLane];
+    route_load_planes<kRouteMaxPerLane>(planes + row, plane_stride, splits, num_experts, bias, logits + row, l);
+    route_compute<kRouteMaxPerLane>(l, num_experts, top_k, e_all, sel_i, sel_w);
+  }
+  if (lane < top_k) {
+    topk_ids[(size_t)t * top_k + lane] = sel_i;
+    topk_weights[(size_t)t * top_k + lane] = sel_w;
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // Dispatch tables (crates/xabe-cuda/src/kernels/moe.rs:2233-2366; CPU:
 // crates/xabe-kernels/src/moe/dispatch.rs:60-131).  Two launches of num_experts workgroups.
@@ -239,6 +268,31 @@ __global__ void __launch_bounds__(256) k_align_scatter(const int* __restrict__ t
 }
 
 // ---------------------------------------------------------------------------------
+// Token-tile lists of the matrix-core grouped GEMM, written by the dispatch kernels below that hold every expert's
+// count and first slot in one workgroup (otherwise by k_build_tiles in mfma.hip, which documents the layout): one
+// entry {expert, first slot, live rows, 0} per `bm`-slot piece of each active expert's run, [0] = the entry count.
+// With bm_b > 0 a second list of that tile height goes to list_b.  bm = 0: no lists asked for.
+// ---------------------------------------------------------------------------------
+struct TileListArgs {
+  int capacity;  // entries a list holds
+  int bm, bm_b;
+  int* list;
+  int* list_b;
+};
+// entries of expert e (count selections from slot `base`), the first of them entry `first` of the list
+__device__ __forceinline__ void write_tile_entries(int e, int count, int base, int first, int h, int capacity, int* list) {
+  const int nt = (count + h - 1) / h;
+  for (int i = 0; i < nt; ++i) {
+    const int idx = first + i;
+    if (idx >= capacity) break;
+    list[4 + 4 * idx + 0] = e;
+    list[4 + 4 * idx + 1] = base + i * h;
+    list[4 + 4 * idx + 2] = min(h, count - i * h);
+    list[4 + 4 * idx + 3] = 0;
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // The same tables from ONE launch of one workgroup, for passes of at most 8192 selections (1024 tokens of top-8):
 // the two launches above cost ~15 us at 512 tokens, nearly all of it launch and barrier latency (every expert's
 // workgroup walks all selections, two barriers per 256 of them).  Sixteen wavefronts split the selections into
@@ -253,10 +307,11 @@ __global__ void __launch_bounds__(1024) k_align_fused(const int* __restrict__ to
                                                        int top_k, int num_experts, int block_size, int sorted_capacity,
                                                        int expert_capacity, int* __restrict__ sorted_token_ids,
                                                        int* __restrict__ expert_ids, int* __restrict__ bucket_live,
-                                                       int* __restrict__ expert_counts, int* __restrict__ num_tokens_post_pad) {
+                                                       int* __restrict__ expert_counts, int* __restrict__ num_tokens_post_pad,
+                                                       TileListArgs tl) {
   constexpr int kMaxE = 512, kRounds = kAlignFusedMaxSelections / (kAlignFusedWaves * 64);
   __shared__ int cnt[kAlignFusedWaves][kMaxE];  // per range and expert: count, then next slot
-  __shared__ int s_scan[2][kMaxE];
+  __shared__ int s_scan[2][3][kMaxE];           // scanned together: padded counts, tiles of either list
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int numel = min(*valid_tokens * top_k, kAlignFusedMaxSelections);
   // whole-capacity fill first: the barriers below order it before the entries written over it
@@ -278,7 +333,7 @@ __global__ void __launch_bounds__(1024) k_align_fused(const int* __restrict__ to
     if (id[r] >= 0) atomicAdd(&cnt[wave][id[r]], 1);
   }
   __syncthreads();
-  int count = 0, padded = 0;
+  int count = 0, padded = 0, tiles_a = 0, tiles_b = 0;
   if (tid < kMaxE) {
     if (tid < num_experts) {
 #pragma unroll
@@ -289,19 +344,32 @@ __global__ void __launch_bounds__(1024) k_align_fused(const int* __restrict__ to
       }
       padded = (count + block_size - 1) / block_size * block_size;
     }
-    s_scan[0][tid] = padded;
+    tiles_a = tl.bm > 0 ? (count + tl.bm - 1) / tl.bm : 0;
+    tiles_b = tl.bm_b > 0 ? (count + tl.bm_b - 1) / tl.bm_b : 0;
+    s_scan[0][0][tid] = padded;
+    s_scan[0][1][tid] = tiles_a;
+    s_scan[0][2][tid] = tiles_b;
   }
   __syncthreads();
   int cur = 0;
   for (int d = 1; d < kMaxE; d <<= 1) {
-    if (tid < kMaxE) s_scan[cur ^ 1][tid] = s_scan[cur][tid] + (tid >= d ? s_scan[cur][tid - d] : 0);
+    if (tid < kMaxE) {
+#pragma unroll
+      for (int a = 0; a < 3; ++a) s_scan[cur ^ 1][a][tid] = s_scan[cur][a][tid] + (tid >= d ? s_scan[cur][a][tid - d] : 0);
+    }
     cur ^= 1;
     __syncthreads();
   }
   if (tid < kMaxE) {
-    const int base = s_scan[cur][tid] - padded;
-    if (tid == kMaxE - 1) *num_tokens_post_pad = s_scan[cur][tid];
+    const int base = s_scan[cur][0][tid] - padded;
+    if (tid == kMaxE - 1) {
+      *num_tokens_post_pad = s_scan[cur][0][tid];
+      if (tl.bm > 0) tl.list[0] = min(s_scan[cur][1][tid], tl.capacity);
+      if (tl.bm_b > 0) tl.list_b[0] = min(s_scan[cur][2][tid], tl.capacity);
+    }
     if (tid < num_experts) {
+      if (tl.bm > 0) write_tile_entries(tid, count, base, s_scan[cur][1][tid] - tiles_a, tl.bm, tl.capacity, tl.list);
+      if (tl.bm_b > 0) write_tile_entries(tid, count, base, s_scan[cur][2][tid] - tiles_b, tl.bm_b, tl.capacity, tl.list_b);
       expert_counts[tid] = count;
 #pragma unroll
       for (int w = 0; w < kAlignFusedWaves; ++w) cnt[w][tid] += base;
@@ -386,9 +454,9 @@ __global__ void __launch_bounds__(512) k_align_offsets(const int* __restrict__ v
                                                         int block_size, int n_chunks_max, int expert_capacity,
                                                         int* __restrict__ chunk_hist, int* __restrict__ expert_counts,
                                                         int* __restrict__ expert_ids, int* __restrict__ bucket_live,
-                                                        int* __restrict__ num_tokens_post_pad) {
+                                                        int* __restrict__ num_tokens_post_pad, TileListArgs tl) {
   static_assert(kAlignMaxExperts == 512, "one thread per expert slot of the scan");
-  __shared__ int s_scan[2][kAlignMaxExperts];
+  __shared__ int s_scan[2][3][kAlignMaxExperts];  // scanned together: padded counts, tiles of either list
   const int e = threadIdx.x;
   const int numel = *valid_tokens * top_k;
   const int n_chunks = min(n_chunks_max, (numel + kAlignChunk - 1) / kAlignChunk);
@@ -402,18 +470,29 @@ __global__ void __launch_bounds__(512) k_align_offsets(const int* __restrict__ v
   if (live)
     for (int c = kAlignCachedChunks; c < n_chunks; ++c) count += chunk_hist[(size_t)c * num_experts + e];
   const int padded = live ? (count + block_size - 1) / block_size * block_size : 0;
-  // inclusive scan of the padded counts (nine doubling steps), then exclusive
-  s_scan[0][e] = padded;
+  const int tiles_a = tl.bm > 0 ? (count + tl.bm - 1) / tl.bm : 0;
+  const int tiles_b = tl.bm_b > 0 ? (count + tl.bm_b - 1) / tl.bm_b : 0;
+  // inclusive scan of the padded counts and the tile counts (nine doubling steps), then exclusive
+  s_scan[0][0][e] = padded;
+  s_scan[0][1][e] = tiles_a;
+  s_scan[0][2][e] = tiles_b;
   __syncthreads();
   int cur = 0;
   for (int d = 1; d < kAlignMaxExperts; d <<= 1) {
-    s_scan[cur ^ 1][e] = s_scan[cur][e] + (e >= d ? s_scan[cur][e - d] : 0);
+#pragma unroll
+    for (int a = 0; a < 3; ++a) s_scan[cur ^ 1][a][e] = s_scan[cur][a][e] + (e >= d ? s_scan[cur][a][e - d] : 0);
     cur ^= 1;
     __syncthreads();
   }
-  const int base = s_scan[cur][e] - padded;
-  if (e == kAlignMaxExperts - 1) *num_tokens_post_pad = s_scan[cur][e];
+  const int base = s_scan[cur][0][e] - padded;
+  if (e == kAlignMaxExperts - 1) {
+    *num_tokens_post_pad = s_scan[cur][0][e];
+    if (tl.bm > 0) tl.list[0] = min(s_scan[cur][1][e], tl.capacity);
+    if (tl.bm_b > 0) tl.list_b[0] = min(s_scan[cur][2][e], tl.capacity);
+  }
   if (!live) return;
+  if (tl.bm > 0) write_tile_entries(e, count, base, s_scan[cur][1][e] - tiles_a, tl.bm, tl.capacity, tl.list);
+  if (tl.bm_b > 0) write_tile_entries(e, count, base, s_scan[cur][2][e] - tiles_b, tl.bm_b, tl.capacity, tl.list_b);
   expert_counts[e] = count;
   int run = base;
 #pragma unroll

@@ -264,6 +264,78 @@ def test_wide_block_passes_back_to_back_keep_their_own_shared_rows(oracle, X):
             assert torch.equal(blk.shared_ungated().view(torch.int32), alone["b"][1]), f"replay {rep}, shared rows"
 
 
+@pytest.mark.parametrize("tokens,biased", [(512, True), (512, False), (2048, True)])
+def test_block_routes_from_the_planes_as_the_step_by_step_calls_do(oracle, X, tokens, biased):
+    """Where the router GEMM splits its contraction, the block adds the partial planes (and the logit bias) in the
+    routing launch instead of a launch of their own.  Same additions in the same order: the logits, the selections
+    and the weights the block leaves are the bits of router_logits + add_logit_bias + route called one by one."""
+    import torch
+
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(tokens), tokens)
+    layer = make_layer(oracle, g, seed=712)
+    x = activations(45, tokens, 2048)
+    bias = torch.from_numpy(_zipf_bias(256, 7, c=1.5)).cuda() if biased else None
+    blk = X.MoeBlock(g)
+    run_block(blk, layer, x, tokens, logit_bias=bias)
+    k = X.MoeKernels(g)
+    b = k.buffers()
+    k.set_valid_tokens(b, tokens)
+    logits = torch.zeros(tokens, 256, device="cuda")
+    k.router_logits(b, layer.dev.router, layer.dev.router_quant, blk.normed(), logits)
+    if biased:
+        k.add_logit_bias(b, bias, logits)
+    k.route(b, logits)
+    torch.cuda.synchronize()
+    assert torch.equal(blk.router_logits().view(torch.int32).reshape(tokens, 256), logits.view(torch.int32))
+    assert torch.equal(blk.buffers().topk_ids(), b.topk_ids())
+    assert torch.equal(blk.buffers().topk_weights().view(torch.int32), b.topk_weights().view(torch.int32))
+
+
+def test_forward_captured_alone_makes_its_own_tile_lists(oracle, X):
+    """The dispatch build leaves the grouped GEMM's token-tile lists, cut for the tile heights of the count then
+    published; a forward trusts them only when both were launched eagerly or recorded into the same capture.  A
+    forward captured on its own carries its own list build: replayed after a wider pass was published and dispatched
+    outside the graph (lists cut for taller tiles), it still gives the bits of the eager forward of that pass."""
+    import torch
+
+    T = 8192
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
+    layer = make_layer(oracle, g, seed=733)
+    d = layer.dev
+    rng = np.random.default_rng(12)
+    logits = torch.from_numpy(rng.uniform(-3, 3, (T, 256)).astype(np.float32)).cuda()
+    x = activations(37, T, 2048)
+    k = X.MoeKernels(g)
+    b = k.buffers()
+    out = torch.zeros(T, 2048, device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        k.set_valid_tokens(b, 512)
+        k.route_and_dispatch(b, logits)
+        k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)       # warm-up of the 64-row form
+        stream.synchronize()
+        small = out[:512].view(torch.int32).clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)   # the forward alone, 64-row tiles
+        out.zero_()
+        graph.replay()
+        stream.synchronize()
+        assert torch.equal(out[:512].view(torch.int32), small)
+        # a full pass, published and dispatched eagerly: the lists the dispatch leaves are cut for 128 / 384 rows
+        k.set_valid_tokens(b, T)
+        k.route_and_dispatch(b, logits)
+        k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)
+        stream.synchronize()
+        wide = out.view(torch.int32).clone()
+        assert torch.equal(wide[:512], small)            # a token's routed row does not depend on the pass's width
+        out.zero_()
+        k.route_and_dispatch(b, logits)                  # (lists for the tall tiles again)
+        graph.replay()                                   # 64-row kernels over the full pass, from their own lists
+        stream.synchronize()
+        assert torch.equal(out.view(torch.int32), wide)
+
+
 @pytest.mark.parametrize("router_q8", [True, False])
 def test_router_logits_matrix_core_path(oracle, X, router_q8):
     # from 2048 tokens up the router runs on the fp32 matrix instruction: fp32 operands, so the logits agree
