@@ -24,10 +24,12 @@ namespace xabe {
 typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr int kRgM = 64;        // tokens per tile
-constexpr int kRgN = 128;       // experts per tile
+constexpr int kRgN = 128;       // experts per tile (64 while the wider tiles are fewer than the compute units)
 constexpr int kRgK = 32;        // contraction step: one Q8_0 block per row
 constexpr int kRgLdA = kRgM + 1;  // LDS tiles are k-major: element (k, m) at k * ld + m
 constexpr int kRgLdB = kRgN + 1;
+// Narrow tiles, 64 experts (each wavefront 32 x 32): twice the workgroups and half the matrix instructions in each.  At
+// 512 tokens the 16 wide tiles in 8 parts are 128 workgroups of ~8 us of fp32 matrix work on 256 compute units.
 
 struct RouterGemmArgs {
   const void* router;   // [E][H] f32, or Q8_0 blocks
@@ -38,13 +40,16 @@ struct RouterGemmArgs {
   int splits, max_tokens;
 };
 
-// grid: (E / 128, ceil(max_tokens / 64), splits); 4 wavefronts as 2 (tokens) x 2 (experts), each 32 x 64.
-template <bool Q8>
+// grid: (E / RN, ceil(max_tokens / 64), splits); 4 wavefronts as 2 (tokens) x 2 (experts), each 32 x RN / 2.
+template <bool Q8, int RN = kRgN>
 __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
+  static_assert(RN == 128 || RN == 64, "expert tile");
+  constexpr int NJ = RN / 64;      // 32-column blocks per wavefront
+  constexpr int kBPer = RN / 8;    // elements of the B tile a thread stages per step
   __shared__ float sA[kRgK * kRgLdA];
   __shared__ float sB[kRgK * kRgLdB];
   const int valid = *a.valid_tokens;
-  const int m0 = blockIdx.y * kRgM, n0 = blockIdx.x * kRgN;
+  const int m0 = blockIdx.y * kRgM, n0 = blockIdx.x * RN;
   if (m0 >= valid) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -52,19 +57,19 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
   // re-read the last live one (computed, never stored)
   const int am = tid >> 2, ak = (tid & 3) * 8;
   const float* arow = a.normed + (size_t)min(m0 + am, valid - 1) * a.H + ak;
-  // B staging: thread -> (expert row tid / 2, sixteen elements at (tid % 2) * 16)
-  const int bn = tid >> 1, bk = (tid & 1) * 16;
+  // B staging: thread -> (expert row tid / 2, sixteen elements at (tid % 2) * 16); narrow tile: row tid / 4, eight
+  const int bn = tid / (32 / kBPer), bk = (tid % (32 / kBPer)) * kBPer;
   const size_t brow_bytes = Q8 ? (size_t)(a.H / 32) * kQ8Bytes : (size_t)a.H * 4;
   const uint8_t* brow = static_cast<const uint8_t*>(a.router) + (size_t)(n0 + bn) * brow_bytes;
 
-  float16v acc[2];
+  float16v acc[NJ];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) acc[j] = (float16v)(0.0f);
+  for (int j = 0; j < NJ; ++j) acc[j] = (float16v)(0.0f);
 
   const int nks_all = a.H / kRgK, ks0 = (int)blockIdx.z * (nks_all / a.splits), nks = ks0 + nks_all / a.splits;
   float* const plane = a.logits + (size_t)blockIdx.z * a.max_tokens * a.E;
   float4 ra[2];
-  float rb[16];
+  float rb[kBPer];
   auto load_step = [&](int ks) {
     ra[0] = reinterpret_cast<const float4*>(arow + (size_t)ks * kRgK)[0];
     ra[1] = reinterpret_cast<const float4*>(arow + (size_t)ks * kRgK)[1];
@@ -74,7 +79,7 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
       const float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(blk));
       const uint16_t* q = reinterpret_cast<const uint16_t*>(blk + 2 + bk);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kBPer / 2; ++i) {
         const uint32_t two = q[i];
         rb[2 * i] = (float)(int8_t)(two & 0xff) * d;
         rb[2 * i + 1] = (float)(int8_t)(two >> 8) * d;
@@ -82,7 +87,7 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
     } else {
       const float4* p = reinterpret_cast<const float4*>(brow + ((size_t)ks * kRgK + bk) * 4);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < kBPer / 4; ++i) {
         const float4 v = p[i];
         rb[4 * i] = v.x; rb[4 * i + 1] = v.y; rb[4 * i + 2] = v.z; rb[4 * i + 3] = v.w;
       }
@@ -95,18 +100,20 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) sA[(ak + i) * kRgLdA + am] = va[i];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) sB[(bk + i) * kRgLdB + bn] = rb[i];
+    for (int i = 0; i < kBPer; ++i) sB[(bk + i) * kRgLdB + bn] = rb[i];
     __syncthreads();
     if (ks + 1 < nks) load_step(ks + 1);  // in flight while the matrix core works
     // operand layout of the 32x32x2 instruction: lane l supplies row (column) l % 32 at k = l / 32
     const float* pa = &sA[(lane >> 5) * kRgLdA + wm * 32 + (lane & 31)];
-    const float* pb = &sB[(lane >> 5) * kRgLdB + wn * 64 + (lane & 31)];
+    const float* pb = &sB[(lane >> 5) * kRgLdB + wn * (RN / 2) + (lane & 31)];
 #pragma unroll
     for (int kk = 0; kk < kRgK / 2; ++kk) {
       const float av = pa[kk * 2 * kRgLdA];
-      const float b0 = pb[kk * 2 * kRgLdB], b1 = pb[kk * 2 * kRgLdB + 32];
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[1], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const float bv = pb[kk * 2 * kRgLdB + 32 * j];
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[j], 0, 0, 0);
+      }
     }
   }
   // acc[j][v]: tile row (v / 4) * 8 + (lane / 32) * 4 + v % 4, column lane % 32 of column block j
@@ -115,7 +122,7 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
     const int t = m0 + wm * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
     if (t >= valid) continue;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) plane[(size_t)t * a.E + n0 + wn * 64 + j * 32 + (lane & 31)] = acc[j][v];
+    for (int j = 0; j < NJ; ++j) plane[(size_t)t * a.E + n0 + wn * (RN / 2) + j * 32 + (lane & 31)] = acc[j][v];
   }
 }
 
@@ -160,9 +167,16 @@ int launch_router_gemm(const xabe_moe_kernels* k, hipStream_t s, const xabe_moe_
   a.valid_tokens = b->valid_tokens;
   a.H = (int)g.hidden;
   a.E = (int)g.num_experts;
-  dim3 grid((unsigned)(g.num_experts / kRgN), (unsigned)((g.max_tokens + kRgM - 1) / kRgM), (unsigned)a.splits);
-  if (router_quant < 0) hipLaunchKernelGGL(k_router_gemm<false>, grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(k_router_gemm<true>, grid, dim3(256), 0, s, a);
+  const size_t m_tiles = (g.max_tokens + kRgM - 1) / kRgM;
+  const bool narrow = g.num_experts / kRgN * m_tiles * a.splits < (size_t)k->num_cus;
+  dim3 grid((unsigned)(g.num_experts / (narrow ? 64 : kRgN)), (unsigned)m_tiles, (unsigned)a.splits);
+  if (narrow) {
+    if (router_quant < 0) hipLaunchKernelGGL((k_router_gemm<false, 64>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_router_gemm<true, 64>), grid, dim3(256), 0, s, a);
+  } else {
+    if (router_quant < 0) hipLaunchKernelGGL((k_router_gemm<false, kRgN>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_router_gemm<true, kRgN>), grid, dim3(256), 0, s, a);
+  }
   XABE_HIP_TRY(hipGetLastError());
   if (a.splits > 1 && sum_deferred) {
     *sum_deferred = true;  // the caller's routing launch adds the planes (k_route_planes)

@@ -337,6 +337,30 @@ def test_forward_captured_alone_makes_its_own_tile_lists(oracle, X):
 
 
 @pytest.mark.parametrize("router_q8", [True, False])
+def test_router_gemm_tile_widths_give_the_same_bits(oracle, X, router_q8):
+    """While its 128-expert tiles are fewer than the compute units (512 tokens) the router GEMM runs 64-expert tiles;
+    a logit is the same products added in the same order either way, so a row of a 512-token pass is the bits it
+    has in a 2048-token pass (128-expert tiles, the contraction in the same eight parts)."""
+    import torch
+
+    g_small = X.MoeGeometry.qwen3_6(X.moe_block_size(512), 512)
+    g_wide = X.MoeGeometry.qwen3_6(X.moe_block_size(2048), 2048)
+    layer = make_layer(oracle, g_small, seed=716, router_q8=router_q8)
+    normed_w = activations(34, 2048, 2048)
+    normed_s = normed_w[:512].clone()
+    out = []
+    for g, normed in ((g_small, normed_s), (g_wide, normed_w)):
+        k = X.MoeKernels(g)
+        b = k.buffers()
+        k.set_valid_tokens(b, g.max_tokens)
+        logits = torch.zeros(g.max_tokens, 256, device="cuda")
+        k.router_logits(b, layer.dev.router, layer.dev.router_quant, normed, logits)
+        torch.cuda.synchronize()
+        out.append(logits)
+    assert torch.equal(out[0].view(torch.int32), out[1][:512].view(torch.int32))
+
+
+@pytest.mark.parametrize("router_q8", [True, False])
 def test_router_logits_matrix_core_path(oracle, X, router_q8):
     # from 2048 tokens up the router runs on the fp32 matrix instruction: fp32 operands, so the logits agree
     # with the CPU reference to fp32 reassociation (the decode-width kernel's bound), for live rows only
