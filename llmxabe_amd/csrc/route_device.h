@@ -38,32 +38,6 @@ __device__ __forceinline__ void route_load(const float* lg, int num_experts, con
   }
 }
 
-// route_load for logits that are still the `splits` (at most 8) partial planes of a split contraction, `plane_stride`
-// floats apart: the planes are added in part order and the bias (may be null) after them, as the stand-alone sum
-// does, and the finished logits are written to `lg_out`.
-template <int PER>
-__device__ __forceinline__ void route_load_planes(const float* planes, size_t plane_stride, int splits, int num_experts,
-                                                  const float* __restrict__ bias, float* lg_out, float (&l)[PER]) {
-  const int lane = threadIdx.x & 63;
-#pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const int idx = i * 64 + lane;
-    l[i] = -INFINITY;
-    if (idx < num_experts) {
-      float part[8];
-#pragma unroll
-      for (int z = 0; z < 8; ++z) part[z] = z < splits ? planes[(size_t)z * plane_stride + idx] : 0.0f;
-      float s = part[0];
-#pragma unroll
-      for (int z = 1; z < 8; ++z)
-        if (z < splits) s += part[z];
-      if (bias) s += bias[idx];
-      lg_out[idx] = s;
-      l[i] = s;
-    }
-  }
-}
-
 // One selection round over per-lane keys (kTaken = out of the running): the largest key, the lowest index
 // among equals; the winner is marked taken.  Returns the winning key and index to every lane.
 // Almost always exactly one (lane, slot) holds the maximum: then its index is read straight off the ballots and
