@@ -815,8 +815,9 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   // (the allocation holds two lists of the same capacity: the down launch's, and the gate/up launch's where its tile
   // height differs)
   const size_t list_ints = b->n_tile_list / 2;
-  int bm, bm_up, cap;
-  (void)mfma_tile_plan(k, b, &bm, &bm_up, &cap);
+  int bm = 0, bm_up = 0, cap = 0;
+  if (!mfma_tile_plan(k, b, &bm, &bm_up, &cap))
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "grouped_forward: these buffers hold no token-tile lists");
   int* list_up = bm_up == bm ? b->tile_list : b->tile_list + list_ints;
   // (the dispatch build has usually left the lists, cut for these heights)
   unsigned long long capture = 0;
