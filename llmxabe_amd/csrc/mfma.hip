@@ -223,7 +223,7 @@ static __device__ long long g_mfma_trace[512 * 32 * 4];
 // instead of two or three, one unit per thread and step instead of two.  A wavefront multiplies only the 32-row
 // blocks that hold live rows, and only live rows' activation pieces are requested.
 template <int QUANT, int NM, bool ROUTED, int TBM = 128>
-__global__ void __launch_bounds__(TBM == 384 ? 512 : 256, 2) k_mfma_expert(MfmaArgs a) {
+__global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_mfma_expert(MfmaArgs a) {
   static_assert(TBM == 384 || TBM == 128 || TBM == 64, "token tile");
   constexpr bool kTall = TBM == 384;
   // Routed tiles are rarely full (an expert's run ends inside its last tile, and below ~1000 tokens most experts hold
@@ -366,13 +366,14 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, 2) k_mfma_expert(MfmaA
       if constexpr (kSkip) {
         if (!(arow_live & (1u << i))) continue;  // (a dead row's slot in LDS keeps whatever it held: its products are dropped)
       }
-      const _Float16* src = a.a + ((size_t)arow_off[i] + (size_t)ks * kBK);
+      // (the tile's base in scalar registers plus a 32-bit byte offset per lane: one address register instead of two)
+      const uint32_t voff = (arow_off[i] + (uint32_t)ks * (uint32_t)kBK) * 2u;
       const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_a + (uint32_t)(kThreads * 16) * i);  // + 16 * lane, by the hardware
       // (m0 is named as clobbered so that the compiler sets it again before any use of its own; it warns that it
       // does not preserve the register across the statement, which is what is wanted here)
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(dst) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(a.a), "s"(dst) : "memory", "m0");
 #pragma clang diagnostic pop
     }
   };
@@ -706,6 +707,10 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
   if (!ok(gate_q) || !ok(down_q) || gate_q != up_q) return false;
   // contraction in steps of 128 (whole Q6_K superblocks: 256); gate/up tiles 64 columns, down tiles 128
   if (g.hidden % 256 != 0 || g.intermediate % 256 != 0) return false;
+  // an activation piece is addressed by a 32-bit byte offset from its tensor's base (fp16 rows of either width, as
+  // many as the sorted table has slots)
+  const size_t rows = g.max_tokens * g.experts_per_token + g.num_experts * g.block_size;
+  if (rows * std::max(g.hidden, g.intermediate) >= ((size_t)1 << 31)) return false;
   return true;
 }
 
