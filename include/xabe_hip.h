@@ -227,6 +227,14 @@ int xabe_moe_add_logit_bias(const xabe_moe_kernels* k, void* stream, const xabe_
  * (crates/xabe-cuda/src/kernels/dequant.rs:19-27). `out` holds blocks*block_elements floats. */
 int xabe_dequantize(void* stream, int quant, const void* bytes, size_t len, float* out, size_t out_len);
 
+/* MmaKernels::quantize_rows (crates/xabe-cuda/src/kernels/mma.rs:769-811, kernel :118-157): fp32 rows [rows][k] ->
+ * int8 `q` [rows][k] and one fp32 scale per 32 elements `scales` [rows][k / 32]; d = amax / 127 (1.0 for a block
+ * of zeros), q = rintf(v * (127 / amax)) clamped to +-127.  Lengths are checked as "at least", as the reference
+ * does; k not a multiple of 32 is XABE_ERR_MMA (MmaError::RaggedContraction).  The matrix-core path of this
+ * library takes fp16 operands and does not use it. */
+int xabe_mma_quantize_rows(void* stream, const float* x, size_t x_len, int8_t* q, size_t q_len, float* scales,
+                           size_t scales_len, size_t rows, size_t k);
+
 /* ---- MoeBlock / MoeLayerWeights (B:634-1330) and DenseFfnBlock (D:1047-1178): block sequencing ---- */
 typedef struct xabe_moe_block xabe_moe_block;
 

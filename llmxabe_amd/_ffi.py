@@ -111,6 +111,7 @@ _SIGNATURES = {
     "xabe_dense_ffn_add_residual": (C.c_int, [vp] * 6),
     "xabe_moe_add_logit_bias": (C.c_int, [vp] * 5),
     "xabe_dequantize": (C.c_int, [vp, C.c_int, vp, sz, vp, sz]),
+    "xabe_mma_quantize_rows": (C.c_int, [vp, vp, sz, vp, sz, vp, sz, sz, sz]),
     "xabe_moe_block_new": (C.c_int, [C.POINTER(Geometry), C.c_float, vp, C.POINTER(vp)]),
     "xabe_moe_block_free": (None, [vp]),
     "xabe_moe_block_publish_tokens": (C.c_int, [vp, vp, sz]),

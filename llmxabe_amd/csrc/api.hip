@@ -1075,6 +1075,25 @@ int xabe_dequantize(void* stream, int quant, const void* bytes, size_t len, floa
   return XABE_OK;
 }
 
+int xabe_mma_quantize_rows(void* stream, const float* x, size_t x_len, int8_t* q, size_t q_len, float* scales,
+                           size_t scales_len, size_t rows, size_t k) {
+  if (!x || !q || !scales) return set_error(XABE_ERR_INVALID_ARGUMENT, "quantize_rows: null pointer");
+  if (k % 32 != 0)
+    return set_error(XABE_ERR_MMA, "contraction length %zu is not a multiple of 32, the elements one scale covers", k);
+  // (at least, as the reference checks them: a caller may quantise the live rows of a larger buffer)
+  const struct { const char* what; size_t have, need; } lens[] = {
+      {"quantize x", x_len, rows * k}, {"quantize q", q_len, rows * k}, {"quantize scales", scales_len, rows * k / 32}};
+  for (const auto& l : lens)
+    if (l.have < l.need)
+      return set_error(XABE_ERR_BUFFER_LENGTH, "%s holds %zu elements, the shape implies %zu", l.what, l.have, l.need);
+  const size_t n_blocks = rows * k / 32;
+  if (n_blocks == 0) return XABE_OK;
+  hipLaunchKernelGGL(k_quantize_rows_q8, dim3((unsigned)((n_blocks + 7) / 8)), dim3(256), 0, as_stream(stream), x, n_blocks, q,
+                     scales);
+  XABE_HIP_TRY(hipGetLastError());
+  return XABE_OK;
+}
+
 // ------------------------------------------------------------------ synthetic stacks
 int xabe_synth_normal_f32(void* stream, uint64_t seed, size_t n, float sigma, float* out) {
   if (!out) return set_error(XABE_ERR_INVALID_ARGUMENT, "synth_normal_f32: null pointer");

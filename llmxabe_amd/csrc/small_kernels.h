@@ -708,6 +708,30 @@ __global__ void __launch_bounds__(256) k_dequant_q8_0(const uint8_t* __restrict_
 }
 
 // ---------------------------------------------------------------------------------
+// Activation rows narrowed to int8 with one fp32 scale per 32 elements, the operand the reference's integer
+// tensor-core path makes before its matmuls (crates/xabe-cuda/src/kernels/mma.rs:118-157): a = max |v| of the block,
+// d = a / 127 (1.0 for a block of zeros), q = rintf(v * (127 / a)) clamped to +-127.  This library multiplies fp16
+// operands instead and never calls it; it is here so that a caller that keeps the int8 form of its activations (or
+// measures against it) finds the reference's values bit for bit.  Half a wavefront per block, one element per lane.
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) k_quantize_rows_q8(const float* __restrict__ x, size_t n_blocks,
+                                                           int8_t* __restrict__ q, float* __restrict__ scales) {
+  const size_t block = (size_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+  if (block >= n_blocks) return;
+  const int lane = threadIdx.x & 31;
+  const float v = x[block * 32 + lane];
+  float a = fabsf(v);
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) a = fmaxf(a, __shfl_xor(a, off, 64));  // (stays inside the 32-lane half)
+  const float d = a > 0.0f ? a / 127.0f : 1.0f;
+  const float inv = a > 0.0f ? 127.0f / a : 0.0f;
+  int qi = (int)rintf(v * inv);
+  qi = qi < -127 ? -127 : (qi > 127 ? 127 : qi);
+  q[block * 32 + lane] = (int8_t)qi;
+  if (lane == 0) scales[block] = d;
+}
+
+// ---------------------------------------------------------------------------------
 // Synthetic stacks: one thread per 256-element chunk.  Integer Irwin-Hall(12) normal
 // approximation over a per-chunk xorshift64* stream, then the reference's amax
 // quantizers (crates/xabe-kernels/src/quant.rs:75-88, :495-567).

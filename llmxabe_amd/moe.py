@@ -293,6 +293,16 @@ class LayerOpsKernels:
                                        out.numel(), rows, width, eps))
 
 
+class MmaKernels:
+    """crates/xabe-cuda/src/kernels/mma.rs:729-811 (quantize_rows only: the matrix-core path here multiplies fp16
+    operands and has no use for the int8 form)."""
+
+    @staticmethod
+    def quantize_rows(x: torch.Tensor, q: torch.Tensor, scales: torch.Tensor, rows: int, k: int):
+        check(_ffi.lib().xabe_mma_quantize_rows(_stream(), _ptr(x), x.numel(), _ptr(q), q.numel(), _ptr(scales),
+                                                scales.numel(), rows, k))
+
+
 def dequantize(quant: ExpertQuant, data: torch.Tensor) -> torch.Tensor:
     """crates/xabe-cuda/src/kernels/dequant.rs: bit-identical to the CPU reference."""
     n = data.numel() // max(1, ExpertQuant(quant).block_bytes()) * ExpertQuant(quant).block_elements()

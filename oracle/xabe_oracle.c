@@ -26,7 +26,8 @@
  *                                            zero weight => zero (gemm.rs:154-266); float64 numpy bound
  *   xo_compare           K/compare.rs:67-135 hand cases
  *   xo_sorted_capacity.. xabe-cuda kernels/moe.rs:4556-4598  reference-held values (moe.rs:6921-6989), brute force
- *   xo_quantize_rows_q8  xabe-cuda kernels/mma.rs:118-157  invariants only
+ *   xo_quantize_rows_q8  xabe-cuda kernels/mma.rs:118-157  closed forms (exact factor, ties to even, zero and
+ *                                            negative blocks), numpy restatement
  *   xo_moe_block_forward xabe-engine block/moe.rs:12-25  composition order: PARITY UNPINNED except by algebraic
  *                                            self-checks ((ffn_out-routed)/shexp == gate, l_out-ffn_out == residual);
  *                                            the reference's behavioural pin is a llama.cpp capture that is not

@@ -255,3 +255,43 @@ def test_geometry_and_error_paths(X):
         k.route(so, torch.zeros(4 * 256, device="cuda"))
     with pytest.raises(X.moe.BufferLength):
         k.route(b, torch.zeros(3 * 256, device="cuda"))
+
+
+def test_quantize_rows_q8_is_the_reference_s_bytes(oracle, X):
+    """MmaKernels::quantize_rows (crates/xabe-cuda/src/kernels/mma.rs:769-811): int8 codes and fp32 scales equal the
+    CPU restatement's bit for bit, on random rows, on blocks of zeros (scale 1.0, codes 0), on values that land
+    exactly between two codes (rintf: ties to even) and on a block whose largest value is negative; lengths are
+    checked as at-least, a ragged contraction is refused."""
+    import torch
+
+    rng = np.random.default_rng(77)
+    rows, k = 37, 2048
+    x = rng.normal(0, 1.5, (rows, k)).astype(np.float32)
+    x[3, 64:96] = 0.0                                   # a block of zeros
+    x[5, :32] = np.arange(32, dtype=np.float32) * 0.5   # amax 15.5: v * (127 / 15.5) hits .5 ties for some v
+    x[5, 31] = 127.0 * 0.25                             # amax 31.75 -> inv = 4: 0.5 * j * 4 = 2 j exactly; and ties:
+    x[5, 1] = 0.125                                     # 0.125 * 4 = 0.5 -> rounds to 0 (even)
+    x[5, 2] = 0.375                                     # 1.5 -> 2
+    x[5, 3] = 0.625                                     # 2.5 -> 2
+    x[7, 32:64] = -np.abs(x[7, 32:64]) - 1.0            # every value negative
+    want_q, want_s = oracle.quantize_rows_q8(x)
+    xd = torch.from_numpy(x).cuda()
+    q = torch.zeros(rows, k, dtype=torch.int8, device="cuda")
+    sc = torch.zeros(rows, k // 32, dtype=torch.float32, device="cuda")
+    X.MmaKernels.quantize_rows(xd, q, sc, rows, k)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), want_q.reshape(rows, k))
+    assert np.array_equal(sc.cpu().numpy().view(np.uint32), want_s.reshape(rows, k // 32).view(np.uint32))
+    got = q.cpu().numpy()
+    assert np.all(got[3, 64:96] == 0) and float(sc[3, 2]) == 1.0
+    assert list(got[5, 1:4]) == [0, 2, 2] and got[5, 31] == 127
+    assert got[7, 32:64].min() == -127
+    # the live rows of a larger buffer: only the first rows are written
+    q.fill_(5)
+    X.MmaKernels.quantize_rows(xd, q, sc, 2, k)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy()[:2], want_q.reshape(rows, k)[:2]) and bool((q[2:] == 5).all())
+    with pytest.raises(X.MoeError, match="not a multiple of 32"):
+        X.MmaKernels.quantize_rows(xd, q, sc, rows, 2040)
+    with pytest.raises(X.MoeError, match="quantize scales holds"):
+        X.MmaKernels.quantize_rows(xd, q, sc[:4], rows, k)

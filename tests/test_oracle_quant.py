@@ -221,3 +221,28 @@ def test_quantize_rows_q8_invariants(oracle):
     assert np.abs(q).max() == 127
     back = q.astype(np.float32).reshape(4, 2, 32) * s[:, :, None]
     assert np.abs(back.reshape(4, 64) - x).max() <= s.max() / 2 + 1e-6
+
+
+def test_quantize_rows_q8_closed_forms(oracle):
+    """xabe-cuda kernels/mma.rs:118-157 on blocks whose answer is known without the code: with amax = 31.75 the
+    factor 127 / amax is exactly 4, so v = j / 8 gives 4 v = j / 2 and rintf's ties go to the even code; a block whose
+    only non-zero is negative puts -127 there; the scale is amax / 127 in fp32; a numpy restatement agrees on random
+    rows (a dropped clamp, truncation instead of rintf, or amax without the absolute value each fail one of these)."""
+    x = np.zeros((2, 64), np.float32)
+    x[0, :32] = np.arange(32, dtype=np.float32) / 8.0
+    x[0, 31] = 31.75
+    x[1, 40] = -2.5
+    q, s = oracle.quantize_rows_q8(x)
+    assert s[0, 0] == np.float32(31.75) / np.float32(127.0)
+    assert list(q[0, :8]) == [0, 0, 1, 2, 2, 2, 3, 4]            # 0, .5, 1, 1.5, 2, 2.5, 3, 3.5 -> ties to even
+    assert q[0, 31] == 127
+    assert s[0, 1] == 1.0 and not q[0, 32:].any()
+    assert q[1, 40] == -127 and s[1, 1] == np.float32(2.5) / np.float32(127.0) and np.count_nonzero(q[1]) == 1
+    r = oracle.Xorshift64Star(21).vec_f32(8 * 256, -4.0, 4.0).reshape(8, 256)
+    q, s = oracle.quantize_rows_q8(r)
+    blocks = r.reshape(8, 8, 32)
+    amax = np.abs(blocks).max(axis=2)
+    inv = (np.float32(127.0) / amax).astype(np.float32)
+    want = np.clip(np.rint((blocks * inv[:, :, None]).astype(np.float32)), -127, 127).astype(np.int8)
+    assert np.array_equal(q.reshape(8, 8, 32), want)
+    assert np.array_equal(s, (amax / np.float32(127.0)).astype(np.float32))
