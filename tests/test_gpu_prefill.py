@@ -264,6 +264,34 @@ def test_wide_block_passes_back_to_back_keep_their_own_shared_rows(oracle, X):
             assert torch.equal(blk.shared_ungated().view(torch.int32), alone["b"][1]), f"replay {rep}, shared rows"
 
 
+def test_block_routes_512_experts_from_the_planes(oracle, X):
+    """The same with 512 experts (eight logits per lane of the routing wavefront, the widest it holds) on the small
+    test shape: logits, selections and weights of the block are the bits of the step-by-step calls, and the
+    selections are the CPU reference's on those logits."""
+    import torch
+
+    tokens = 256
+    g = X.MoeGeometry(512, 4, 512, 256, 32, tokens)
+    layer = make_layer(oracle, g, seed=719)
+    x = activations(46, tokens, 512)
+    bias = torch.from_numpy(_zipf_bias(512, 11, c=1.0)).cuda()
+    blk = X.MoeBlock(g)
+    run_block(blk, layer, x, tokens, logit_bias=bias)
+    k = X.MoeKernels(g)
+    b = k.buffers()
+    k.set_valid_tokens(b, tokens)
+    logits = torch.zeros(tokens, 512, device="cuda")
+    k.router_logits(b, layer.dev.router, layer.dev.router_quant, blk.normed(), logits)
+    k.add_logit_bias(b, bias, logits)
+    k.route(b, logits)
+    torch.cuda.synchronize()
+    assert torch.equal(blk.router_logits().view(torch.int32).reshape(tokens, 512), logits.view(torch.int32))
+    assert torch.equal(blk.buffers().topk_ids(), b.topk_ids())
+    assert torch.equal(blk.buffers().topk_weights().view(torch.int32), b.topk_weights().view(torch.int32))
+    ids = blk.buffers().topk_ids().cpu().numpy().reshape(tokens, 4)
+    assert np.array_equal(ids, oracle.route_batch(logits.cpu().numpy(), 4)[0].astype(np.int32))
+
+
 @pytest.mark.parametrize("tokens,biased", [(512, True), (512, False), (2048, True)])
 def test_block_routes_from_the_planes_as_the_step_by_step_calls_do(oracle, X, tokens, biased):
     """Where the router GEMM splits its contraction, the block adds the partial planes (and the logit bias) in the
