@@ -293,8 +293,7 @@ def main() -> int:
     # ---- the prefill half of the metric: the 8192-token chunk (MFMA-bound) and configs[2]'s 512-token chunk under a
     # seeded Zipf(1.1) router bias (HBM-bound), on the first layers of the same weight sets ----
     if not args.no_prefill:
-        rank = np.random.default_rng(5).permutation(256) + 1
-        zipf = torch.from_numpy((-1.1 * np.log(rank)).astype(np.float32)).cuda()
+        zipf = torch.from_numpy(X.zipf_logit_bias(256)).cuda()
         out["prefill"] = {"tokens_8192": prefill_leg(X, layers[:2], 8192, 20),
                           "tokens_512_zipf": prefill_leg(X, layers[:4], 512, 40, bias=zipf)}
         out["prefill"]["mfma_util_pct"] = 100.0 * out["prefill"]["tokens_8192"]["frac_of_mfma_peak"]
@@ -424,8 +423,7 @@ def other_workload(args) -> int:
     if args.workload == "prefill_512":
         # the skewed configuration: a seeded Zipf(s = 1.1) bias over the experts, added to the router logits before
         # routing (b_e = -s ln(rank_e) over a seeded permutation of the experts, i.e. selection odds proportional to rank^-1.1)
-        rank = np.random.default_rng(5).permutation(256) + 1
-        extra["logit_bias"] = torch.from_numpy((-1.1 * np.log(rank)).astype(np.float32)).cuda()
+        extra["logit_bias"] = torch.from_numpy(X.zipf_logit_bias(256)).cuda()
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()
     reps_w = max(1, min(args.warmup, 64) // L)

@@ -285,7 +285,8 @@ int xabe_moe_block_tensor_cores_enabled(const xabe_moe_block* blk);      /* B:10
  * formats of the three-launch decode block; anything larger is XABE_ERR_UNSUPPORTED_GEOMETRY.  The live-token count
  * is published by a one-thread kernel, so the call may be captured.  All calls on one GPU share that GPU's array:
  * calls that overlap on one GPU race.  The first call on a device resolves the array's address there; make it
- * outside a capture. */
+ * outside a capture (a first call that arrives while `stream` is capturing is refused with
+ * XABE_ERR_INVALID_ARGUMENT and records nothing). */
 int xabe_moe_block_forward_noalloc(const xabe_moe_geometry* geometry, float eps, void* stream,
                                    const xabe_moe_layer_weights* w, const float* residual, size_t residual_len,
                                    size_t tokens, const float* logit_bias, float* ffn_out, size_t ffn_out_len, float* l_out,

@@ -573,9 +573,8 @@ int xabe_moe_set_valid_tokens(const xabe_moe_kernels* k, void* stream, xabe_moe_
   // A change of the count is a host-to-device copy, and a copy recorded into a graph would publish, on every replay,
   // whatever the source holds then.  Like the reference (kernels/moe.rs:5473-5491: "callable outside graph capture"),
   // the count is set before a capture begins; a call that would change it inside one is refused, with nothing recorded.
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  XABE_HIP_TRY(hipStreamIsCapturing(as_stream(stream), &capturing));
-  if (capturing != hipStreamCaptureStatusNone)
+  // (a query the runtime refuses is read as "not capturing": the copy below then reports what it has to)
+  if (stream_capture_id(as_stream(stream)) != 0 && stream_capture_id(as_stream(stream)) != kCaptureUnknown)
     return set_error(XABE_ERR_INVALID_ARGUMENT,
                      "set_valid_tokens: the stream is capturing and the live-token count would change from %d to %zu; "
                      "publish the count before the capture begins",
@@ -614,7 +613,8 @@ int xabe_moe_build_dispatch(const xabe_moe_kernels* k, void* stream, xabe_moe_bu
   TileListArgs tl;
   memset(&tl, 0, sizeof(tl));
   b->tiles_bm = b->tiles_bm_up = 0;
-  XABE_TRY(stream_capture_id(s, &b->tiles_capture));
+  b->tiles_capture = stream_capture_id(s);
+  if (b->tiles_capture != 0) b->tiles_graph_owned = true;
   int bm = 0, bm_up = 0, cap = 0;
   const bool lists = mfma_tile_plan(k, b, &bm, &bm_up, &cap) && g.num_experts <= 512;
   if (lists) {

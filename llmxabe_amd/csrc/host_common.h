@@ -40,13 +40,19 @@ int validate_geometry(const xabe_moe_geometry& g);  // MoeKernels::new's checks 
   } while (0)
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
-// id of the capture `s` is recording into, 0 when it is not capturing
-inline int stream_capture_id(hipStream_t s, unsigned long long* id) {
+// id of the capture `s` is recording into, 0 when it is not capturing.  A query the runtime refuses (the legacy
+// stream while another stream of the process captures in global mode) is not an error of the caller's: it answers
+// kCaptureUnknown, which compares unequal to every capture and to "eager", and clears the runtime's error state.
+// Handles are meant for explicit streams.
+constexpr unsigned long long kCaptureUnknown = ~0ull;
+inline unsigned long long stream_capture_id(hipStream_t s) {
   hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
   unsigned long long cid = 0;
-  XABE_HIP_TRY(hipStreamGetCaptureInfo(s, &status, &cid));
-  *id = status == hipStreamCaptureStatusActive ? cid : 0;
-  return XABE_OK;
+  if (hipStreamGetCaptureInfo(s, &status, &cid) != hipSuccess) {
+    (void)hipGetLastError();
+    return kCaptureUnknown;
+  }
+  return status == hipStreamCaptureStatusActive ? cid : 0;
 }
 
 }  // namespace xabe
@@ -166,6 +172,10 @@ struct xabe_moe_buffers {
   // eagerly after an eager build, so that a captured forward never depends on lists made outside its graph
   int tiles_bm, tiles_bm_up;
   unsigned long long tiles_capture;
+  // set for good once a dispatch build on these buffers has been recorded into a capture: a replay of that graph
+  // rewrites the device lists without touching the fields above, so from then on only a forward inside a capture
+  // that holds its own build trusts them; eager forwards always make their own
+  bool tiles_graph_owned;
   float* router_partial;  // [split][token][expert]: the router GEMM's contraction splits at mid widths
   size_t n_router_partial;
   size_t bytes;

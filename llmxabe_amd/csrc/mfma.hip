@@ -825,9 +825,12 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
     return set_error(XABE_ERR_INVALID_ARGUMENT, "grouped_forward: these buffers hold no token-tile lists");
   int* list_up = bm_up == bm ? b->tile_list : b->tile_list + list_ints;
   // (the dispatch build has usually left the lists, cut for these heights)
-  unsigned long long capture = 0;
-  XABE_TRY(stream_capture_id(s, &capture));
-  if (b->tiles_bm != bm || b->tiles_bm_up != bm_up || b->tiles_capture != capture) {
+  // trusted only when nothing can have rewritten them since: inside the capture that holds the build, or eagerly
+  // after an eager build on buffers no graph has ever recorded a build on
+  const unsigned long long capture = stream_capture_id(s);
+  const bool trusted = b->tiles_bm == bm && b->tiles_bm_up == bm_up && capture != kCaptureUnknown &&
+                       b->tiles_capture == capture && (capture != 0 || !b->tiles_graph_owned);
+  if (!trusted) {
     hipLaunchKernelGGL(k_build_tiles, dim3(1), dim3(256), 0, s, b->expert_counts, (int)g.num_experts, (int)g.block_size, cap,
                        bm, b->tile_list, bm_up != bm ? bm_up : 0, list_up);
     XABE_HIP_TRY(hipGetLastError());

@@ -43,8 +43,10 @@ constexpr int kNaMaxDevices = 64;
 static std::mutex g_na_mutex;
 static float* g_na_ptr[kNaMaxDevices];  // the array's address on each device, resolved on first use there
 
-// The calling thread's current device and the address of that device's copy of the array.
-static int na_scratch(float** out) {
+// The calling thread's current device and the address of that device's copy of the array.  The address is resolved
+// on the first call on a device, and that call must not arrive while `s` is capturing: resolving the symbol may load
+// the code object, which a capture in progress does not survive; such a call is refused with nothing recorded.
+static int na_scratch(hipStream_t s, float** out) {
   int dev = 0;
   XABE_HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kNaMaxDevices)
@@ -52,6 +54,10 @@ static int na_scratch(float** out) {
                      dev, kNaMaxDevices);
   std::lock_guard<std::mutex> lock(g_na_mutex);
   if (!g_na_ptr[dev]) {
+    if (stream_capture_id(s) != 0)
+      return set_error(XABE_ERR_INVALID_ARGUMENT,
+                       "block_forward_noalloc: the first call on device %d arrived while the stream is capturing; make one "
+                       "call on the device before the capture begins", dev);
     float* p = nullptr;
     XABE_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)));
     if (!p) return set_error(XABE_ERR_DRIVER, "block_forward_noalloc: the scratch array has no address on device %d", dev);
@@ -93,7 +99,7 @@ int xabe_moe_block_forward_noalloc(const xabe_moe_geometry* geometry, float eps,
   if (l_out_len != n_act) return set_error(XABE_ERR_BUFFER_LENGTH, "l_out holds %zu elements, expected %zu", l_out_len, n_act);
 
   float* base = nullptr;
-  XABE_TRY(na_scratch(&base));
+  XABE_TRY(na_scratch(as_stream(stream), &base));
 
   // host-side views over the scratch array, in the shape the launch code takes the block's buffers in
   xabe_moe_kernels k;

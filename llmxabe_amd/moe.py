@@ -317,6 +317,20 @@ def synth_normal_f32(seed: int, n: int, sigma: float) -> torch.Tensor:
     return out
 
 
+ZIPF_BIAS_SEED = 5   # the skewed-routing workload's permutation of the experts
+
+
+def zipf_logit_bias(num_experts: int, seed: int = ZIPF_BIAS_SEED, s: float = 1.1, c: float = 1.0):
+    """The skewed-routing workload's per-expert logit bias, b_e = -c * s * ln(rank_e) with rank a seeded permutation
+    of 1..num_experts (selection odds proportional to rank^(-c*s)); a host float32 array.  The reference has no bias
+    input: a harness adds it to the logits between the router GEMV and `route`.  One definition for the benchmark and
+    the parity tests, so that what is timed is what is checked."""
+    import numpy as np
+
+    rank = np.random.default_rng(seed).permutation(num_experts) + 1
+    return (-c * s * np.log(rank)).astype(np.float32)
+
+
 def calibrate_hbm_read(buffer: torch.Tensor, sink: torch.Tensor) -> None:
     """One launch that reads every 16-byte piece of `buffer` once, coalesced; the caller times it."""
     check(_ffi.lib().xabe_calibrate_hbm_read(_stream(), _ptr(buffer), buffer.numel() * buffer.element_size(), _ptr(sink)))

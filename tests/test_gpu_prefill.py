@@ -90,22 +90,25 @@ def test_grouped_forward_small_geometry(oracle, X, fmt, max_tokens, tokens, mode
     assert rel_to_peak(out2.cpu().numpy()[:tokens], ref) <= 2e-5
 
 
-def _zipf_bias(num_experts, seed, s=1.1, c=1.0):
-    """b_e = c * log(1 / rank_e^s) over a seeded permutation of the experts."""
-    rank = np.random.default_rng(seed).permutation(num_experts) + 1
-    return (-c * s * np.log(rank)).astype(np.float32)
+# (layer seed, activations seed, c of the Zipf bias): "benched" is bench.py's `tokens_512_zipf` leg on its first
+# layer (layer seed 10000, activations seed 99, b_e = -1.1 ln rank_e), input for input; "steep" a harsher skew
+PREFILL_512_CASES = {"uniform": (710, 32, None), "benched": (10000, 99, 1.0), "steep": (710, 32, 2.0)}
 
 
-@pytest.mark.parametrize("tokens,skew", [(512, False), (512, True)])
-def test_block_prefill_512_matches_oracle(oracle, X, tokens, skew):
-    """BASELINE configs[2]: a 512-token chunk; with skew=True a Zipf(1.1) bias on the router logits, so a
-    few experts receive 50+ tokens and many receive none."""
+@pytest.mark.parametrize("case", sorted(PREFILL_512_CASES))
+def test_block_prefill_512_matches_oracle(oracle, X, case):
+    """BASELINE configs[2]: a 512-token chunk; the skewed cases put a seeded Zipf(1.1) bias on the router logits
+    (`llmxabe_amd.zipf_logit_bias`, the definition bench.py times), so a few experts receive 50+ tokens and many
+    receive none."""
     import torch
 
+    tokens = 512
+    layer_seed, x_seed, c = PREFILL_512_CASES[case]
+    skew = c is not None
     g = X.MoeGeometry.qwen3_6(X.moe_block_size(tokens), tokens)
-    layer = make_layer(oracle, g, seed=710)
-    x = activations(32, tokens, 2048)
-    bias_np = _zipf_bias(256, 5, c=2.0) if skew else None
+    layer = make_layer(oracle, g, seed=layer_seed)
+    x = activations(x_seed, tokens, 2048)
+    bias_np = X.zipf_logit_bias(256, c=c) if skew else None
     bias = torch.from_numpy(bias_np).cuda() if skew else None
     blk = X.MoeBlock(g)
     ffn_out, l_out = run_block(blk, layer, x, tokens, logit_bias=bias)
@@ -274,7 +277,7 @@ def test_block_routes_512_experts_from_the_planes(oracle, X):
     g = X.MoeGeometry(512, 4, 512, 256, 32, tokens)
     layer = make_layer(oracle, g, seed=719)
     x = activations(46, tokens, 512)
-    bias = torch.from_numpy(_zipf_bias(512, 11, c=1.0)).cuda()
+    bias = torch.from_numpy(X.zipf_logit_bias(512, seed=11)).cuda()
     blk = X.MoeBlock(g)
     run_block(blk, layer, x, tokens, logit_bias=bias)
     k = X.MoeKernels(g)
@@ -302,7 +305,7 @@ def test_block_routes_from_the_planes_as_the_step_by_step_calls_do(oracle, X, to
     g = X.MoeGeometry.qwen3_6(X.moe_block_size(tokens), tokens)
     layer = make_layer(oracle, g, seed=712)
     x = activations(45, tokens, 2048)
-    bias = torch.from_numpy(_zipf_bias(256, 7, c=1.5)).cuda() if biased else None
+    bias = torch.from_numpy(X.zipf_logit_bias(256, seed=7, c=1.5)).cuda() if biased else None
     blk = X.MoeBlock(g)
     run_block(blk, layer, x, tokens, logit_bias=bias)
     k = X.MoeKernels(g)
@@ -360,6 +363,57 @@ def test_forward_captured_alone_makes_its_own_tile_lists(oracle, X):
         out.zero_()
         k.route_and_dispatch(b, logits)                  # (lists for the tall tiles again)
         graph.replay()                                   # 64-row kernels over the full pass, from their own lists
+        stream.synchronize()
+        assert torch.equal(out.view(torch.int32), wide)
+
+
+def test_eager_forward_after_a_replayed_dispatch_graph_makes_its_own_tile_lists(oracle, X):
+    """The other direction: a graph that holds a dispatch build rewrites the device's tile lists on every replay without
+    the host knowing.  Capture the dispatch of a full pass (lists cut for 128 / 384 rows), then publish 512 tokens and
+    dispatch eagerly (the host now believes the lists are cut for 64 rows), replay the graph, and run the forward
+    eagerly: it must not run the 64-row kernels over the graph's tall entries."""
+    import torch
+
+    T = 8192
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
+    layer = make_layer(oracle, g, seed=734)
+    d = layer.dev
+    rng = np.random.default_rng(13)
+    logits = torch.from_numpy(rng.uniform(-3, 3, (T, 256)).astype(np.float32)).cuda()
+    x = activations(38, T, 2048)
+    k = X.MoeKernels(g)
+    b = k.buffers()
+    out = torch.zeros(T, 2048, device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        # reference rows of the full pass, all eager
+        k.set_valid_tokens(b, T)
+        k.route_and_dispatch(b, logits)
+        k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)
+        stream.synchronize()
+        wide = out.view(torch.int32).clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            k.route_and_dispatch(b, logits)              # the dispatch alone: tall lists on every replay
+        graph.replay()
+        # a 512-token pass dispatched eagerly: 64-row lists, and the host's bookkeeping says so
+        k.set_valid_tokens(b, 512)
+        k.route_and_dispatch(b, logits)
+        k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)
+        stream.synchronize()
+        assert torch.equal(out[:512].view(torch.int32), wide[:512])
+        # the graph rewrites tables and lists for whatever count is published (512 here) at the heights it was captured for
+        out.zero_()
+        graph.replay()
+        k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)
+        stream.synchronize()
+        assert torch.equal(out[:512].view(torch.int32), wide[:512])
+        assert not out[512:].any()
+        # and the full pass through the same sequence
+        k.set_valid_tokens(b, T)
+        out.zero_()
+        graph.replay()
+        k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)
         stream.synchronize()
         assert torch.equal(out.view(torch.int32), wide)
 
