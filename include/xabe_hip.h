@@ -260,6 +260,46 @@ int xabe_moe_block_publish_tokens(xabe_moe_block* blk, void* stream, size_t toke
 int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
                            size_t residual_len, size_t tokens, const float* logit_bias, float* ffn_out,
                            size_t ffn_out_len, float* l_out, size_t l_out_len);
+/* The post-mixer seam between consecutive layers (the reference's seam-fusion work, docs/BENCHMARKS.md:1340-1377 and
+ * the row it measured at :1761, "the next layer's RMSNorm in the MoE combine kernel's tail ... the mixer skips its
+ * norm launch").  Two halves that pair up across a layer boundary:
+ *   producer: with `next_norm_weight` set, the launch that finishes l_out also writes
+ *             next_normed = rms_norm(l_out, next_norm_weight, next_eps) for the live rows (and, if `next_normed_h` is
+ *             set, the same values rounded once to fp16, the copy the matrix-core kernels read), so the consumer of
+ *             l_out launches no RMSNorm and makes no second pass over l_out;
+ *   consumer: with `input_normed` nonzero, the block takes its normalised rows as given in its own `normed` buffer
+ *             (xabe_moe_block_normed_mut; at matrix-core widths also the fp16 copy, xabe_moe_block_normed_h_mut)
+ *             instead of normalising `residual`, which it still adds back at the end.
+ * Every tensor holds the bits the unfused sequence (block, RMSNorm launch, block) produces; rows past the live
+ * count of next_normed are left as they were.  next_normed may be the producing block's own normed buffer (one
+ * handle serving every layer of a stack).  Hidden sizes above 2048 take the separate RMSNorm launch inside the call.
+ * `ffn_out` may be NULL here (a read-back tensor the layer loop does not consume); with `skip_readback` nonzero the
+ * `routed` tensor behind xabe_moe_block_routed is not written either (its contents are then stale). */
+typedef struct xabe_moe_seam {
+  int input_normed;
+  int skip_readback;
+  const float* next_norm_weight; /* [hidden] or NULL */
+  float next_eps;
+  float* next_normed;            /* [max_tokens][hidden] */
+  size_t next_normed_len;
+  void* next_normed_h;           /* fp16 [max_tokens][hidden] or NULL */
+  size_t next_normed_h_len;
+} xabe_moe_seam;
+/* xabe_moe_block_forward with a seam on either side; `seam` NULL is xabe_moe_block_forward itself. */
+int xabe_moe_block_forward_seam(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
+                                size_t residual_len, size_t tokens, const float* logit_bias, float* ffn_out,
+                                size_t ffn_out_len, float* l_out, size_t l_out_len, const xabe_moe_seam* seam);
+/* Writable views of the block's normalised rows for a producer's `next_normed` / `next_normed_h` (the second is NULL
+ * with length 0 below matrix-core widths, where no kernel reads an fp16 copy). */
+float* xabe_moe_block_normed_mut(xabe_moe_block* blk, size_t* len);
+void* xabe_moe_block_normed_h_mut(xabe_moe_block* blk, size_t* len);
+/* The combine with the producer half of the seam as a step of its own, for callers that sequence the block
+ * themselves (xabe_moe_gate_and_combine plus the tail; `routed` and `ffn_out` may be NULL; the next_* arguments as in
+ * xabe_moe_seam, all NULL for the plain combine).  Rows of at most 2048 elements. */
+int xabe_moe_gate_and_combine_seam(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b,
+                                   const float* shared_gate_inp, const float* normed, const float* shexp,
+                                   const float* residual, float* gate, float* routed, float* ffn_out, float* l_out,
+                                   const float* next_norm_weight, float next_eps, float* next_normed, void* next_normed_h);
 int xabe_moe_block_disable_tensor_cores(xabe_moe_block* blk);            /* B:987-989 */
 int xabe_moe_block_set_exact_decode_regime(xabe_moe_block* blk, int on); /* B:1003-1005 */
 /* At max_tokens <= 32 and the model shapes (hidden 2048 / intermediate 512, and the 512 / 256 test shape) the

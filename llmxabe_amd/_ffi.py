@@ -34,6 +34,11 @@ class MoeLayerWeightsC(C.Structure):
                 ("shared_gate", QuantTensorC), ("shared_up", QuantTensorC), ("shared_down", QuantTensorC)]
 
 
+class SeamC(C.Structure):
+    _fields_ = [("input_normed", C.c_int), ("skip_readback", C.c_int), ("next_norm_weight", vp), ("next_eps", C.c_float),
+                ("next_normed", vp), ("next_normed_len", sz), ("next_normed_h", vp), ("next_normed_h_len", sz)]
+
+
 class DenseLayerWeightsC(C.Structure):
     _fields_ = [("post_norm", vp), ("gate", QuantTensorC), ("up", QuantTensorC), ("down", QuantTensorC)]
 
@@ -116,6 +121,10 @@ _SIGNATURES = {
     "xabe_moe_block_free": (None, [vp]),
     "xabe_moe_block_publish_tokens": (C.c_int, [vp, vp, sz]),
     "xabe_moe_block_forward": (C.c_int, [vp, vp, C.POINTER(MoeLayerWeightsC), vp, sz, sz, vp, vp, sz, vp, sz]),
+    "xabe_moe_block_forward_seam": (C.c_int, [vp, vp, C.POINTER(MoeLayerWeightsC), vp, sz, sz, vp, vp, sz, vp, sz, C.POINTER(SeamC)]),
+    "xabe_moe_block_normed_mut": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_block_normed_h_mut": (vp, [vp, C.POINTER(sz)]),
+    "xabe_moe_gate_and_combine_seam": (C.c_int, [vp] * 12 + [C.c_float, vp, vp]),
     "xabe_moe_block_forward_noalloc": (C.c_int, [C.POINTER(Geometry), C.c_float, vp, C.POINTER(MoeLayerWeightsC), vp, sz, sz, vp, vp, sz,
                                                  vp, sz]),
     "xabe_moe_block_disable_tensor_cores": (C.c_int, [vp]),

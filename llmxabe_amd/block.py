@@ -12,7 +12,7 @@ from typing import Optional
 import torch
 
 from . import _ffi
-from ._ffi import DenseLayerWeightsC, FfnConfigC, FfnLayerWeightsC, Geometry, MoeLayerWeightsC
+from ._ffi import DenseLayerWeightsC, FfnConfigC, FfnLayerWeightsC, Geometry, MoeLayerWeightsC, SeamC
 from .moe import ExpertQuant, MoeBuffers, MoeGeometry, QuantTensor, _ptr, _stream, _wrap, check
 
 DEFAULT_RMS_EPS = 1e-6  # block/moe.rs:179
@@ -72,6 +72,28 @@ class MoeBlock:
         check(_ffi.lib().xabe_moe_block_forward(self._h, _stream(), C.byref(cw), _ptr(residual), residual.numel(), tokens,
                                                 _ptr(logit_bias), _ptr(ffn_out), ffn_out.numel(), _ptr(l_out),
                                                 l_out.numel()))
+
+    def forward_seam(self, w: MoeLayerWeights, residual, tokens: int, ffn_out, l_out, logit_bias=None, input_normed=False,
+                     next_norm_weight=None, next_block: "MoeBlock | None" = None, next_eps: float | None = None,
+                     skip_readback=False):
+        """`forward` across the post-mixer seam (see the header): with `next_norm_weight`, the launch that finishes
+        l_out also leaves rms_norm(l_out, next_norm_weight) in `next_block`'s normalised-rows buffers (this block's
+        own when `next_block` is None: one handle serving every layer); with `input_normed`, this block starts from
+        the rows a previous call left there.  `ffn_out` may be None."""
+        cw = w._c()
+        seam = SeamC(int(input_normed), int(skip_readback), 0, 0.0, 0, 0, 0, 0)
+        if next_norm_weight is not None:
+            dst = next_block if next_block is not None else self
+            n, nh = C.c_size_t(0), C.c_size_t(0)
+            seam.next_norm_weight = _ptr(next_norm_weight)
+            seam.next_eps = dst._eps if next_eps is None else next_eps
+            seam.next_normed = _ffi.lib().xabe_moe_block_normed_mut(dst._h, C.byref(n))
+            seam.next_normed_len = n.value
+            seam.next_normed_h = _ffi.lib().xabe_moe_block_normed_h_mut(dst._h, C.byref(nh))
+            seam.next_normed_h_len = nh.value
+        check(_ffi.lib().xabe_moe_block_forward_seam(self._h, _stream(), C.byref(cw), _ptr(residual), residual.numel(), tokens,
+                                                     _ptr(logit_bias), _ptr(ffn_out), 0 if ffn_out is None else ffn_out.numel(),
+                                                     _ptr(l_out), l_out.numel(), C.byref(seam)))
 
     def forward_stage(self, w: MoeLayerWeights, residual, ffn_out, l_out, stage: int, logit_bias=None):
         """One of the three decode launches alone (measurement hook; see the header)."""

@@ -520,6 +520,8 @@ static int alloc_buffers(const xabe_moe_kernels* k, void* stream, int scope, boo
                             ? (size_t)router_gemm_splits(g) * g.max_tokens * g.num_experts
                             : 0;
   A(&b->router_partial, b->n_router_partial);
+  // decode widths: one arrival counter per token for the seam's tail in the third launch (decode_block.hip)
+  A(&b->seam_arrivals, (routed && g.max_tokens <= 32) ? g.max_tokens : 0);
   b->bytes = total;
   b->valid_published = 0;
   if (st != XABE_OK) {
@@ -540,7 +542,7 @@ void xabe_moe_buffers_free(xabe_moe_buffers* b) {
   if (!b) return;
   void* ptrs[] = {b->topk_ids, b->topk_weights, b->sorted_token_ids, b->expert_ids, b->bucket_live, b->expert_counts,
                   b->num_tokens_post_pad, b->valid_tokens, b->align_hist, b->inter, b->partial, b->shared_inter, b->x_h, b->inter_h,
-                  b->shared_inter_h, b->tile_list, b->router_partial};
+                  b->shared_inter_h, b->tile_list, b->router_partial, b->seam_arrivals};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   delete b;
@@ -1031,6 +1033,38 @@ int xabe_moe_gate_and_combine(const xabe_moe_kernels* k, void* stream, const xab
   dim3 grid((unsigned)g.max_tokens, (unsigned)((g.hidden + 1023) / 1024));
   hipLaunchKernelGGL(k_gate_and_combine, grid, dim3(256), 0, as_stream(stream), shared_gate_inp, normed, b->partial, shexp,
                      residual, b->valid_tokens, (int)g.experts_per_token, (int)g.hidden, gate, routed, ffn_out, l_out);
+  XABE_HIP_TRY(hipGetLastError());
+  return XABE_OK;
+}
+
+int xabe_moe_gate_and_combine_seam(const xabe_moe_kernels* k, void* stream, const xabe_moe_buffers* b,
+                                   const float* shared_gate_inp, const float* normed, const float* shexp,
+                                   const float* residual, float* gate, float* routed, float* ffn_out, float* l_out,
+                                   const float* next_norm_weight, float next_eps, float* next_normed, void* next_normed_h) {
+  if (!k || !b || !shared_gate_inp || !normed || !shexp || !residual || !gate || !l_out)
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "gate_and_combine_seam: null pointer");
+  XABE_TRY(require_routed(b, "gate_and_combine_seam"));
+  const xabe_moe_geometry& g = k->g;
+  if (g.hidden > 2048)
+    return set_error(XABE_ERR_UNSUPPORTED_GEOMETRY, "gate_and_combine_seam: rows of %zu elements; the one-workgroup-per-row combine serves at most 2048", g.hidden);
+  if (next_norm_weight && !next_normed)
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "gate_and_combine_seam: a norm weight for the next layer but nowhere to write its rows");
+  const uintptr_t align = reinterpret_cast<uintptr_t>(normed) | reinterpret_cast<uintptr_t>(shexp) | reinterpret_cast<uintptr_t>(residual) |
+                          reinterpret_cast<uintptr_t>(routed) | reinterpret_cast<uintptr_t>(ffn_out) | reinterpret_cast<uintptr_t>(l_out) |
+                          reinterpret_cast<uintptr_t>(next_norm_weight) | reinterpret_cast<uintptr_t>(next_normed) |
+                          reinterpret_cast<uintptr_t>(next_normed_h);
+  if (align % 16 != 0) return set_error(XABE_ERR_INVALID_ARGUMENT, "gate_and_combine_seam: tensors must be 16-byte aligned");
+  const dim3 grid((unsigned)g.max_tokens);
+  hipStream_t s = as_stream(stream);
+  _Float16* nh = static_cast<_Float16*>(next_normed_h);
+#define XABE_COMBINE(NORM, WITH_H)                                                                                          \
+  hipLaunchKernelGGL((k_combine_rows<NORM, WITH_H>), grid, dim3(256), 0, s, shared_gate_inp, normed, b->partial, shexp,     \
+                     residual, b->valid_tokens, (int)g.experts_per_token, (int)g.hidden, gate, routed, ffn_out, l_out,        \
+                     next_norm_weight, next_eps, next_normed, nh)
+  if (!next_norm_weight) XABE_COMBINE(false, false);
+  else if (nh) XABE_COMBINE(true, true);
+  else XABE_COMBINE(true, false);
+#undef XABE_COMBINE
   XABE_HIP_TRY(hipGetLastError());
   return XABE_OK;
 }

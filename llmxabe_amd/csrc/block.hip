@@ -120,32 +120,63 @@ static int route_rows(xabe_moe_block* blk, void* stream, const xabe_moe_layer_we
 int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
                            size_t residual_len, size_t tokens, const float* logit_bias, float* ffn_out,
                            size_t ffn_out_len, float* l_out, size_t l_out_len) {
-  if (!blk || !w || !residual || !ffn_out || !l_out) return set_error(XABE_ERR_INVALID_ARGUMENT, "MoeBlock::forward: null pointer");
+  if (!ffn_out) return set_error(XABE_ERR_INVALID_ARGUMENT, "MoeBlock::forward: null pointer");
+  return xabe_moe_block_forward_seam(blk, stream, w, residual, residual_len, tokens, logit_bias, ffn_out, ffn_out_len, l_out,
+                                     l_out_len, nullptr);
+}
+
+float* xabe_moe_block_normed_mut(xabe_moe_block* blk, size_t* len) {
+  if (len) *len = blk ? blk->n_act : 0;
+  return blk ? blk->normed : nullptr;
+}
+void* xabe_moe_block_normed_h_mut(xabe_moe_block* blk, size_t* len) {
+  void* p = blk && blk->buffers ? blk->buffers->x_h : nullptr;
+  if (len) *len = p ? blk->n_act : 0;
+  return p;
+}
+
+int xabe_moe_block_forward_seam(xabe_moe_block* blk, void* stream, const xabe_moe_layer_weights* w, const float* residual,
+                                size_t residual_len, size_t tokens, const float* logit_bias, float* ffn_out,
+                                size_t ffn_out_len, float* l_out, size_t l_out_len, const xabe_moe_seam* seam) {
+  if (!blk || !w || !residual || !l_out || (!ffn_out && !seam))
+    return set_error(XABE_ERR_INVALID_ARGUMENT, "MoeBlock::forward: null pointer");
   const xabe_moe_geometry& g = blk->g;
   if (tokens > g.max_tokens)
     return set_error(XABE_ERR_TOO_MANY_TOKENS, "%zu tokens exceeds the %zu the block was sized for", tokens, g.max_tokens);
   XABE_TRY(blk_check_len("residual", blk->n_act, residual_len));
-  XABE_TRY(blk_check_len("ffn_out", blk->n_act, ffn_out_len));
+  if (ffn_out) XABE_TRY(blk_check_len("ffn_out", blk->n_act, ffn_out_len));
   XABE_TRY(blk_check_len("l_out", blk->n_act, l_out_len));
+  const bool pre = seam && seam->input_normed;
+  const bool tail = seam && seam->next_norm_weight;
+  if (tail) {
+    if (!seam->next_normed) return set_error(XABE_ERR_INVALID_ARGUMENT, "MoeBlock::forward: a seam with a norm weight but no next_normed");
+    XABE_TRY(blk_check_len("next_normed", blk->n_act, seam->next_normed_len));
+    if (seam->next_normed_h) XABE_TRY(blk_check_len("next_normed_h", blk->n_act, seam->next_normed_h_len));
+  }
   XABE_TRY(xabe_moe_block_publish_tokens(blk, stream, tokens));
 
   // decode widths, model shapes: the eight steps below regrouped into three launches, same arithmetic
   if (blk->fused_decode && !blk->moe->exact_regime && decode_block_supported(blk->moe, blk->buffers, w)) {
     XABE_TRY(check_layer_stacks(blk->moe, w));  // (the checks the step-by-step sequence below makes call by call)
+    DecodeSeam ds = {pre, tail ? seam->next_norm_weight : nullptr, tail ? seam->next_eps : 0.0f, tail ? seam->next_normed : nullptr,
+                     tail ? seam->next_normed_h : nullptr};
     return launch_decode_block(blk->moe, as_stream(stream), blk->buffers, w, residual, logit_bias, blk->eps, blk->normed,
-                               blk->logits, blk->shexp, blk->gate, blk->routed, ffn_out, l_out);
+                               blk->logits, blk->shexp, blk->gate, blk->routed, ffn_out, l_out, 7u, seam ? &ds : nullptr);
   }
 
   const bool wide = g.max_tokens >= kMfmaMinTokens && xabe_moe_kernels_tensor_cores_enabled(blk->moe);
   // 1. post-mixer RMSNorm over every row of the buffer; at matrix-core widths the same launch writes the fp16 copy
-  //    of the rows that the routed and the shared expert kernels read
-  bool normed_h = false;
-  if (wide && blk->buffers->x_h)
-    XABE_TRY(rms_norm_rows_with_f16(stream, residual, w->post_norm, blk->normed, blk->buffers->x_h, g.max_tokens, g.hidden,
-                                    blk->eps, &normed_h));
-  if (!normed_h)
-    XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
-                           g.hidden, blk->eps));
+  //    of the rows that the routed and the shared expert kernels read.  With the seam's consumer half on, the previous
+  //    block's tail has left both already.
+  bool normed_h = pre && wide && blk->buffers->x_h;
+  if (!pre) {
+    if (wide && blk->buffers->x_h)
+      XABE_TRY(rms_norm_rows_with_f16(stream, residual, w->post_norm, blk->normed, blk->buffers->x_h, g.max_tokens, g.hidden,
+                                      blk->eps, &normed_h));
+    if (!normed_h)
+      XABE_TRY(xabe_rms_norm(stream, residual, blk->n_act, w->post_norm, g.hidden, blk->normed, blk->n_act, g.max_tokens,
+                             g.hidden, blk->eps));
+  }
   const bool shared_mma =
       wide && mfma_supported(blk->moe, blk->buffers, w->shared_gate.quant, w->shared_up.quant, w->shared_down.quant, false);
   if (shared_mma && blk->side) {
@@ -196,9 +227,29 @@ int xabe_moe_block_forward(xabe_moe_block* blk, void* stream, const xabe_moe_lay
       if (st != XABE_OK) return st;
     }
   }
-  // 5. routed sum, sigmoid gate, combine, residual
-  return xabe_moe_gate_and_combine(blk->moe, stream, blk->buffers, w->shared_gate_inp, blk->normed, blk->shexp, residual,
-                                   blk->gate, blk->routed, ffn_out, l_out);
+  // 5. routed sum, sigmoid gate, combine, residual (and, across a seam, the next layer's RMSNorm in the same launch)
+  if (!seam)
+    return xabe_moe_gate_and_combine(blk->moe, stream, blk->buffers, w->shared_gate_inp, blk->normed, blk->shexp, residual,
+                                     blk->gate, blk->routed, ffn_out, l_out);
+  float* routed = seam->skip_readback ? nullptr : blk->routed;
+  if (g.hidden <= 2048)
+    return xabe_moe_gate_and_combine_seam(blk->moe, stream, blk->buffers, w->shared_gate_inp, blk->normed, blk->shexp, residual,
+                                          blk->gate, routed, ffn_out, l_out, tail ? seam->next_norm_weight : nullptr,
+                                          tail ? seam->next_eps : 0.0f, tail ? seam->next_normed : nullptr,
+                                          tail ? seam->next_normed_h : nullptr);
+  // longer rows: the plain combine (which writes every tensor) and the RMSNorm as a launch of its own: the same values
+  if (!ffn_out) return set_error(XABE_ERR_INVALID_ARGUMENT, "MoeBlock::forward: rows of %zu elements take the plain combine, which needs an ffn_out", g.hidden);
+  XABE_TRY(xabe_moe_gate_and_combine(blk->moe, stream, blk->buffers, w->shared_gate_inp, blk->normed, blk->shexp, residual,
+                                     blk->gate, blk->routed, ffn_out, l_out));
+  if (!tail) return XABE_OK;
+  bool with_h = false;
+  if (seam->next_normed_h)
+    XABE_TRY(rms_norm_rows_with_f16(stream, l_out, seam->next_norm_weight, seam->next_normed, seam->next_normed_h, g.max_tokens,
+                                    g.hidden, seam->next_eps, &with_h));
+  if (!with_h)
+    XABE_TRY(xabe_rms_norm(stream, l_out, blk->n_act, seam->next_norm_weight, g.hidden, seam->next_normed, blk->n_act,
+                           g.max_tokens, g.hidden, seam->next_eps));
+  return XABE_OK;
 }
 
 int xabe_moe_block_disable_tensor_cores(xabe_moe_block* blk) {

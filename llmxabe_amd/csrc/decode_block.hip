@@ -100,6 +100,13 @@ struct DecodeArgs {
   float* routed;
   float* ffn_out;
   float* l_out;
+  // the seam to the next layer (all null / zero when the pass ends at l_out): the last workgroup of the third launch to
+  // finish a token's row applies the next layer's RMSNorm to it (arrival counters: one int per token, zero between passes)
+  const float* next_w;
+  float* next_normed;
+  _Float16* next_normed_h;
+  int* arrivals;
+  float next_eps;
   size_t expert_bytes;  // bytes of one expert's gate (= up) matrix
   size_t down_bytes;    // bytes of one expert's down matrix (its format may differ)
   float eps;
@@ -120,7 +127,9 @@ struct DecodeArgs {
 constexpr int kXnPad = kStepElems + kStepElems / 8;  // floats per staged row
 __device__ __forceinline__ int xn_at(int e) { return e + 4 * (e >> 5); }
 
-template <int QUANT, int RPS, int TC, int NM, int D>
+// PRE: the rows handed over are normalised already (the previous block's tail wrote them into this block's `normed`):
+// they are staged and used as they are, no norm weight, no scale.
+template <int QUANT, int RPS, int TC, int NM, int D, bool PRE>
 __device__ __forceinline__ void tile_normed(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1, int K,
                                             int n_rows, int row0, const float* const (&xrow)[TC],
                                             const float* __restrict__ norm_w, float eps, float* const (&out)[TC],
@@ -147,12 +156,13 @@ __device__ __forceinline__ void tile_normed(const uint8_t* __restrict__ w0, cons
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int i = (int)threadIdx.x + 256 * j, ic = min(i, n4 - 1);
-    const float4 nq = reinterpret_cast<const float4*>(norm_w)[ic];
+    float4 nq = make_float4(0.f, 0.f, 0.f, 0.f);
+    if constexpr (!PRE) nq = reinterpret_cast<const float4*>(norm_w)[ic];
     float4 xq[TC];
 #pragma unroll
     for (int t = 0; t < TC; ++t) xq[t] = reinterpret_cast<const float4*>(xrow[t])[ic];
     if (i < n4) {
-      *reinterpret_cast<float4*>(s_nw + xn_at(4 * i)) = nq;
+      if constexpr (!PRE) *reinterpret_cast<float4*>(s_nw + xn_at(4 * i)) = nq;
 #pragma unroll
       for (int t = 0; t < TC; ++t) *reinterpret_cast<float4*>(s_xn + t * kXnPad + xn_at(4 * i)) = xq[t];
     }
@@ -171,12 +181,16 @@ __device__ __forceinline__ void tile_normed(const uint8_t* __restrict__ w0, cons
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int off = QUANT == kQ6K ? koff + g.half * 128 + j * 32 + g.l8 * 8 : koff + j * 8;
-    lds8(s_nw, off, nw, j * 8);
+    if constexpr (!PRE) lds8(s_nw, off, nw, j * 8);
 #pragma unroll
     for (int t = 0; t < TC; ++t) lds8(s_xn + t * kXnPad, off, x[t], j * 8);
   }
 #pragma unroll
   for (int t = 0; t < TC; ++t) {
+    if constexpr (PRE) {
+      lane_x_offsets<QUANT>(x[t], xs[t]);
+      continue;
+    }
     float f[32];
     const int base = g.lane * 32;  // (lanes past the row's end fold zeros: fma(0, 0, s) == s)
 #pragma unroll
@@ -220,7 +234,7 @@ __device__ __forceinline__ void tile_normed(const uint8_t* __restrict__ w0, cons
 // A: grid = max_tokens (norm + gate scalar) + chunks * tiles_r (router) + chunks * tiles_s (shared gate/up).
 // A chunk is two tokens sharing one pass over the weights.
 // ------------------------------------------------------------------------------------------------
-template <int SQ, int RF, int RPS, int kLogitsDepth>
+template <int SQ, int RF, int RPS, int kLogitsDepth, bool PRE = false>
 __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
   __shared__ float s_red[4];
   __shared__ __attribute__((aligned(16))) float s_xn[3 * kXnPad];  // the chunk's rows and the norm weight
@@ -235,24 +249,24 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
     const int tiles = router ? a.tiles_r : a.tiles_s;
     const int c = item / tiles, tile = item % tiles, t0 = 2 * c;
     const int row0 = (tile * kWavesPerWg + wave) * RPS * kLogitsDepth;
-    const float* x0 = a.residual + (size_t)t0 * a.H;
+    const float* x0 = (PRE ? a.normed : a.residual) + (size_t)t0 * a.H;
     if (t0 + 1 < a.max_tokens) {
       const float* const xr[2] = {x0, x0 + a.H};
       if (router) {
         float* const o[2] = {a.logits + (size_t)t0 * a.E, a.logits + (size_t)(t0 + 1) * a.E};
-        tile_normed<RF, RPS, 2, 1, kLogitsDepth>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0, s_xn);
+        tile_normed<RF, RPS, 2, 1, kLogitsDepth, PRE>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0, s_xn);
       } else {
         float* const o[2] = {a.shared_inter + (size_t)t0 * a.I, a.shared_inter + (size_t)(t0 + 1) * a.I};
-        tile_normed<SQ, RPS, 2, 2, kLogitsDepth>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0, s_xn);
+        tile_normed<SQ, RPS, 2, 2, kLogitsDepth, PRE>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0, s_xn);
       }
     } else {
       const float* const xr[1] = {x0};
       if (router) {
         float* const o[1] = {a.logits + (size_t)t0 * a.E};
-        tile_normed<RF, RPS, 1, 1, kLogitsDepth>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0, s_xn);
+        tile_normed<RF, RPS, 1, 1, kLogitsDepth, PRE>(a.router, nullptr, a.H, a.E, row0, xr, a.post_norm, a.eps, o, a.logit_bias, a.valid_tokens, t0, s_xn);
       } else {
         float* const o[1] = {a.shared_inter + (size_t)t0 * a.I};
-        tile_normed<SQ, RPS, 1, 2, kLogitsDepth>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0, s_xn);
+        tile_normed<SQ, RPS, 1, 2, kLogitsDepth, PRE>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0, s_xn);
       }
     }
     XABE_TRACE(0, 3);
@@ -262,7 +276,7 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
   // operations of the stand-alone RMSNorm and gate kernels
   const int t = blockIdx.x;
   const int valid = *a.valid_tokens;
-  const float* xr = a.residual + (size_t)t * a.H;
+  const float* xr = (PRE ? a.normed : a.residual) + (size_t)t * a.H;
   // hidden <= 2048: eight columns per thread, every load issued before the first use
   float xv[8], nv[8], gv[8];
 #pragma unroll
@@ -270,18 +284,22 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
     const int j = threadIdx.x + 256 * i;
     const bool in = j < a.H;
     xv[i] = in ? xr[j] : 0.0f;
-    nv[i] = in ? a.post_norm[j] : 0.0f;
+    nv[i] = in && !PRE ? a.post_norm[j] : 0.0f;
     gv[i] = in ? a.shared_gate_inp[j] : 0.0f;
   }
-  const float inv = row_inv_rms(xr, a.H, a.eps);
+  float inv = 1.0f;
+  if constexpr (!PRE) inv = row_inv_rms(xr, a.H, a.eps);
   if (t >= valid) return;
   float s = 0.0f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int j = threadIdx.x + 256 * i;
     if (j < a.H) {
-      const float v = xv[i] * inv * nv[i];
-      a.normed[(size_t)t * a.H + j] = v;
+      float v = xv[i];  // (PRE: the row is there already, written by the previous block's tail)
+      if constexpr (!PRE) {
+        v = xv[i] * inv * nv[i];
+        a.normed[(size_t)t * a.H + j] = v;
+      }
       s = __builtin_fmaf(gv[i], v, s);
     }
   }
@@ -585,10 +603,56 @@ __global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
     const float v = r + sh * gate;
     a.routed[i] = r;
     a.shexp[i] = sh;
-    a.ffn_out[i] = v;
-    a.l_out[i] = v + a.residual[i];
+    if (a.ffn_out) a.ffn_out[i] = v;
+    const float lo = v + a.residual[i];
+    // (with the seam on, another workgroup of this launch reads the row back: the store goes through to memory)
+    if (a.next_normed) __hip_atomic_store(a.l_out + i, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else a.l_out[i] = lo;
   }
   XABE_TRACE(2, 3);
+  if (!a.next_normed) return;
+  // The seam (docs/BENCHMARKS.md:1376 of the reference: the next layer's RMSNorm in the combine's tail).  A token's
+  // row is finished by tiles_d workgroups; each counts its arrival once its stores have been acknowledged, and the
+  // one that arrives last reads the row back (agent-scope loads: the other workgroups' stores went through to memory,
+  // no fence, whose L2 write-back costs microseconds here), forms the RMS scale in the canonical order and writes
+  // the normalised row: the bits of the stand-alone RMSNorm launch on l_out.
+  __shared__ int s_last;
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (threadIdx.x == 0)
+    s_last = __hip_atomic_fetch_add(a.arrivals + t, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.tiles_d - 1;
+  __syncthreads();
+  if (!s_last || wave != 0) return;
+  if (lane == 0) __hip_atomic_store(a.arrivals + t, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next pass
+  // the row comes in coalesced (element 64 j + lane per load) and changes hands through LDS (s_x is free now), padded
+  // by four floats per 32 as the first launch pads its rows
+  float* s_l = s_x;
+  const float* lrow = a.l_out + (size_t)t * a.H;
+  float in[32];
+#pragma unroll
+  for (int j = 0; j < 32; ++j) {
+    const int e = 64 * j + lane;
+    in[j] = e < a.H ? __hip_atomic_load(lrow + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+  }
+#pragma unroll
+  for (int j = 0; j < 32; ++j) s_l[xn_at(64 * j + lane)] = in[j];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  RmsRaw rowq;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) rowq.q[j] = *reinterpret_cast<const float4*>(s_l + xn_at(32 * lane + 4 * j));
+  const float inv = rms_finish(rms_fold(rowq, 0.0f), a.H, a.next_eps);
+  // out the same way: element 64 j + lane, (x * inv) * w
+#pragma unroll
+  for (int j = 0; j < 32; ++j) {
+    const int e = 64 * j + lane;
+    if (e < a.H) {
+      const float v = in[j] * inv * a.next_w[e];
+      a.next_normed[(size_t)t * a.H + e] = v;
+      if (a.next_normed_h) a.next_normed_h[(size_t)t * a.H + e] = (_Float16)v;
+    }
+  }
 }
 
 // ------------------------------------------------------------------ host side
@@ -597,6 +661,7 @@ struct Launch {
   hipStream_t s;
   unsigned grid_a, grid_b, grid_c;
   bool pre_routed;  // a routing launch between A and B instead of routing inside B
+  bool pre_normed;  // `normed` holds this pass's rows already (the previous block's tail): A neither normalises nor writes them
   size_t route_lds;
   unsigned launches;  // bit i: issue launch i (A, B, C); all three outside measurements
 };
@@ -610,18 +675,24 @@ static bool launch_all(const Launch& l, int gq, int dq, int sgq, int sdq, int ro
   const bool rf32 = router_quant < 0;
   if (!rf32 && router_quant != XABE_QUANT_Q8_0) return false;
   if (l.launches & 1u) {
-#define XABE_A(SQ, RF)                                                                                              \
+#define XABE_A1(SQ, RF, PRE)                                                                                        \
   do {                                                                                                            \
     const int da = logits_depth(l.a.max_tokens);                                                                  \
-    if (da == 1) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 1>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);  \
-    else if (da == 2) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 2>), dim3(l.grid_a), dim3(256), 0, l.s, l.a); \
-    else hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 4>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);          \
+    if (da == 1) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 1, PRE>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);  \
+    else if (da == 2) hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 2, PRE>), dim3(l.grid_a), dim3(256), 0, l.s, l.a); \
+    else hipLaunchKernelGGL((k_decode_logits<SQ, RF, RPSH, 4, PRE>), dim3(l.grid_a), dim3(256), 0, l.s, l.a);     \
+  } while (0)
+#define XABE_A(SQ, RF)                  \
+  do {                                  \
+    if (l.pre_normed) XABE_A1(SQ, RF, true); \
+    else XABE_A1(SQ, RF, false);        \
   } while (0)
     if (sg6 && rf32) XABE_A(kQ6K, kF32);
     else if (sg6) XABE_A(kQ6K, kQ8_0);
     else if (rf32) XABE_A(kQ8_0, kF32);
     else XABE_A(kQ8_0, kQ8_0);
 #undef XABE_A
+#undef XABE_A1
   }
   if (l.launches & 2u) {
     if (l.pre_routed) {
@@ -665,10 +736,20 @@ bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b
 
 int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, const xabe_moe_layer_weights* w,
                         const float* residual, const float* logit_bias, float eps, float* normed, float* logits,
-                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches) {
+                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches,
+                        const DecodeSeam* seam) {
   const xabe_moe_geometry& g = k->g;
   DecodeArgs a;
   memset(&a, 0, sizeof(a));
+  if (seam && seam->next_normed) {
+    if (!b->seam_arrivals)
+      return set_error(XABE_ERR_INVALID_ARGUMENT, "decode block: these buffers carry no arrival counters for the seam");
+    a.next_w = seam->next_w;
+    a.next_normed = seam->next_normed;
+    a.next_normed_h = static_cast<_Float16*>(seam->next_normed_h);
+    a.next_eps = seam->next_eps;
+    a.arrivals = b->seam_arrivals;
+  }
   a.residual = residual;
   a.post_norm = w->post_norm;
   a.router = static_cast<const uint8_t*>(w->router);
@@ -714,7 +795,7 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
                      a.E, a.I, rps_h);
   const int chunks = (a.max_tokens + 1) / 2;
   const bool pre_routed = a.max_tokens >= kPreRouteMinTokens;
-  Launch l{a, s, 0, 0, 0, pre_routed, g.num_experts * sizeof(float), launches};
+  Launch l{a, s, 0, 0, 0, pre_routed, seam && seam->input_normed, g.num_experts * sizeof(float), launches};
   l.grid_a = (unsigned)(chunks * (a.tiles_r + a.tiles_s) + a.max_tokens);
   l.grid_b = (unsigned)(a.max_tokens * a.top_k * a.tiles_g);
   l.grid_c = (unsigned)(a.max_tokens * a.tiles_d);

@@ -74,9 +74,20 @@ bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b
 // the checks the step-by-step entry points make on a layer's six stacks (whole blocks, element counts, formats,
 // 16-byte-aligned device pointers), for the block-level paths that launch without passing through them (api.hip)
 int check_layer_stacks(const xabe_moe_kernels* k, const xabe_moe_layer_weights* w);
+// The seam between this block and the next as the decode launches see it: `input_normed`: `normed` holds the pass's
+// rows already; `next_normed` (null: the pass ends at l_out): where the third launch's last workgroup per token
+// writes rms_norm(l_out, next_w, next_eps), `next_normed_h` (may be null) its fp16 copy.
+struct DecodeSeam {
+  bool input_normed;
+  const float* next_w;
+  float next_eps;
+  float* next_normed;
+  void* next_normed_h;
+};
 int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffers* b, const xabe_moe_layer_weights* w,
                         const float* residual, const float* logit_bias, float eps, float* normed, float* logits,
-                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches = 7u);
+                        float* shexp, float* gate_out, float* routed, float* ffn_out, float* l_out, unsigned launches = 7u,
+                        const DecodeSeam* seam = nullptr);
 
 // matrix-core regime (mfma.hip)
 // dense block, fp32 widths, rows longer than one step: norm + gate/up, down + residual (api.hip)
@@ -176,6 +187,7 @@ struct xabe_moe_buffers {
   // rewrites the device lists without touching the fields above, so from then on only a forward inside a capture
   // that holds its own build trusts them; eager forwards always make their own
   bool tiles_graph_owned;
+  int32_t* seam_arrivals;  // [max_tokens], decode widths: arrival counters of the seam's tail (zero between passes)
   float* router_partial;  // [split][token][expert]: the router GEMM's contraction splits at mid widths
   size_t n_router_partial;
   size_t bytes;

@@ -659,6 +659,107 @@ __global__ void __launch_bounds__(256) k_gate_and_combine(const float* __restric
   *reinterpret_cast<float4*>(l_out + base + j) = lo;
 }
 
+// The same combine for rows of at most 2048 elements, one workgroup per token, with the post-mixer seam fusion the
+// reference measured on its own card ("the next layer's RMSNorm in the MoE combine kernel's tail",
+// docs/BENCHMARKS.md:1376, :1761): the workgroup holds the whole row of l_out, so it can apply the NEXT layer's
+// RMSNorm to it before it leaves, and the next block starts from normalised rows (and, WITH_H, from their fp16 copy)
+// without a launch of its own or a second pass over l_out.  Every value is the one the separate launches produce:
+// gate, routed sum, ffn_out and l_out in k_gate_and_combine's operations and order; the RMS scale of the row in the
+// canonical order (lane L of a wavefront folds elements 32L .. 32L+31, then the wavefront tree: the row changes
+// hands through LDS for that, padded like k_rms_norm_short_rows'), the normalised elements as (x * inv) * w.
+// `routed` and `ffn_out` may be null (read-back tensors a serving loop does not need: 16 bytes per element less
+// to write); NORM = false leaves the tail out.
+template <bool NORM, bool WITH_H>
+__global__ void __launch_bounds__(256) k_combine_rows(const float* __restrict__ w, const float* normed,
+                                                       const float* __restrict__ partial, const float* __restrict__ shexp,
+                                                       const float* __restrict__ residual, const int* __restrict__ valid_tokens,
+                                                       int top_k, int hidden, float* __restrict__ gate,
+                                                       float* __restrict__ routed, float* __restrict__ ffn_out,
+                                                       float* __restrict__ l_out, const float* __restrict__ next_w, float next_eps,
+                                                       float* next_normed, _Float16* __restrict__ next_normed_h) {
+  // (`next_normed` may be `normed` itself, a block that feeds the next pass through its own buffers: the row is read
+  // in round one and written after the last barrier, by this workgroup only)
+  constexpr int kSlots = 512 + 64;  // padded 16-byte slots of one 2048-element row
+  __shared__ float scratch[4];
+  __shared__ float4 s_row[NORM ? kSlots : 1];
+  const int t = blockIdx.x;
+  if (t >= *valid_tokens) return;
+  const size_t base = (size_t)t * hidden;
+  const int n4 = hidden / 4;
+  // round one: everything the row needs, requested together (two 16-byte columns per thread)
+  const float4* p4 = reinterpret_cast<const float4*>(partial + (size_t)t * top_k * hidden);
+  float4 pv[2][8], sh[2], rs[2], nw[2];
+  float wv[8], xv[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int j = min((int)threadIdx.x + 256 * i, hidden - 1);
+    wv[i] = w[j];
+    xv[i] = normed[base + j];
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = min((int)threadIdx.x + 256 * i, n4 - 1);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) pv[i][k] = p4[(size_t)min(k, top_k - 1) * n4 + q];
+    sh[i] = reinterpret_cast<const float4*>(shexp + base)[q];
+    rs[i] = reinterpret_cast<const float4*>(residual + base)[q];
+    if constexpr (NORM) nw[i] = reinterpret_cast<const float4*>(next_w)[q];
+  }
+  // selections past the eighth (top_k > 8) are added from memory in the loop below
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    if ((int)threadIdx.x + 256 * i < hidden) s = __builtin_fmaf(wv[i], xv[i], s);
+  s = block_sum_256(s, scratch);
+  const float g = 1.0f / (1.0f + expf(-s));
+  if (threadIdx.x == 0) gate[t] = g;
+  float4 lo[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = (int)threadIdx.x + 256 * i;
+    lo[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (q < n4) {
+      float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (k < top_k) { r.x += pv[i][k].x; r.y += pv[i][k].y; r.z += pv[i][k].z; r.w += pv[i][k].w; }
+      for (int k = 8; k < top_k; ++k) {
+        const float4 v = p4[(size_t)k * n4 + q];
+        r.x += v.x; r.y += v.y; r.z += v.z; r.w += v.w;
+      }
+      float4 v;
+      v.x = r.x + sh[i].x * g; v.y = r.y + sh[i].y * g; v.z = r.z + sh[i].z * g; v.w = r.w + sh[i].w * g;
+      lo[i].x = v.x + rs[i].x; lo[i].y = v.y + rs[i].y; lo[i].z = v.z + rs[i].z; lo[i].w = v.w + rs[i].w;
+      if (routed) reinterpret_cast<float4*>(routed + base)[q] = r;
+      if (ffn_out) reinterpret_cast<float4*>(ffn_out + base)[q] = v;
+      reinterpret_cast<float4*>(l_out + base)[q] = lo[i];
+    }
+    if constexpr (NORM) s_row[q + (q >> 3)] = lo[i];  // (zeros past the end of a short row: fma(0, 0, s) == s)
+  }
+  if constexpr (NORM) {
+    __syncthreads();
+    const int lane = (int)__lane_id();
+    RmsRaw r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.q[i] = s_row[8 * lane + i + lane];  // slot(8 * lane + i)
+    const float inv = rms_finish(rms_fold(r, 0.0f), hidden, next_eps);  // every wavefront: the same scale
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int q = (int)threadIdx.x + 256 * i;
+      if (q < n4) {
+        const float4 v = make_float4(lo[i].x * inv * nw[i].x, lo[i].y * inv * nw[i].y, lo[i].z * inv * nw[i].z,
+                                     lo[i].w * inv * nw[i].w);
+        reinterpret_cast<float4*>(next_normed + base)[q] = v;
+        if constexpr (WITH_H) {
+          typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+          const h2 a = {(_Float16)v.x, (_Float16)v.y}, b = {(_Float16)v.z, (_Float16)v.w};
+          reinterpret_cast<uint2*>(next_normed_h + base)[q] = make_uint2(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b));
+        }
+      }
+    }
+  }
+}
+
 // dense_ffn_add_residual (crates/xabe-engine/src/block/dense_ffn.rs:1149-1175)
 __global__ void __launch_bounds__(256) k_add_residual(const float* __restrict__ ffn_out, const float* __restrict__ residual,
                                                        const int* __restrict__ valid_tokens, int hidden,

@@ -279,6 +279,15 @@ class MoeKernels:
                                                    _ptr(shexp), _ptr(residual), _ptr(gate), _ptr(routed), _ptr(ffn_out),
                                                    _ptr(l_out)))
 
+    def gate_and_combine_seam(self, buffers, shared_gate_inp, normed, shexp, residual, gate, routed, ffn_out, l_out,
+                              next_norm_weight=None, next_eps: float = 1e-6, next_normed=None, next_normed_h=None):
+        """`gate_and_combine` with the next layer's RMSNorm applied to l_out in the same launch (see the header);
+        `routed` and `ffn_out` may be None."""
+        check(_ffi.lib().xabe_moe_gate_and_combine_seam(self._h, _stream(), buffers._h, _ptr(shared_gate_inp), _ptr(normed),
+                                                        _ptr(shexp), _ptr(residual), _ptr(gate), _ptr(routed), _ptr(ffn_out),
+                                                        _ptr(l_out), _ptr(next_norm_weight), next_eps, _ptr(next_normed),
+                                                        _ptr(next_normed_h)))
+
     def dense_ffn_add_residual(self, buffers, ffn_out, residual, l_out):
         check(_ffi.lib().xabe_dense_ffn_add_residual(self._h, _stream(), buffers._h, _ptr(ffn_out), _ptr(residual),
                                                      _ptr(l_out)))
