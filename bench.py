@@ -116,6 +116,8 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the two prefill legs of the headline run")
     ap.add_argument("--no-calibration", action="store_true", help="skip the read / matrix-instruction calibration legs")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the compact legs of BASELINE's other configurations (decode batch 32, the dense sibling, the 40-layer stack)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--workload", default="decode_b3", choices=["decode_b3"] + sorted(OTHER_WORKLOADS),
                     help="decode_b3 is the headline: the batch-3 decode block (value, roofline), followed by the "
@@ -302,6 +304,25 @@ def main() -> int:
         out["calibration"] = calibration(X, stream)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(layers[0], g, x, T, args.cpu_seconds)
+    # ---- BASELINE's remaining configurations, one compact leg each (the same code `--workload NAME` runs alone):
+    # configs[3] decode batch 32 as a block and through the 40-layer stack, configs[4] the dense sibling ----
+    if not args.no_configs:
+        del layers, x, ffn_out, l_out
+        torch.cuda.empty_cache()
+        legs = {}
+        for name in ("decode_b32", "dense_b1", "dense_b8", "dense_2048", "stack40_b32"):
+            r = run_other(args, name)
+            leg = {"tokens": r["config"]["tokens"], "ms_per_step": r["ms_per_step"], "tokens_per_s": r["value"], "steps": r["steps"],
+                   "algorithmic_bytes_per_step": r["algorithmic_bytes_per_step"], "flops_per_step": r["flops_per_step"],
+                   "bound": r["roofline"]["bound"], "achieved": r["roofline"]["achieved"], "unit": r["roofline"]["unit"],
+                   "frac": r["roofline"]["frac"]}
+            for key in ("layers", "us_per_layer", "layers_rotated", "distinct_experts"):
+                if key in r["config"]:
+                    leg[key] = r["config"][key]
+            if "seam" in r:
+                leg["seam"] = r["seam"]
+            legs[name] = leg
+        out["configs"] = legs
     print(json.dumps(out))
     return 0
 
@@ -375,13 +396,18 @@ MFMA_PEAK_TFLOPS = 2500.0
 OTHER_WORKLOADS = {"decode_b32": ("moe", 32, 16), "prefill_512": ("moe", 512, 4), "prefill_512_uniform": ("moe", 512, 4),
                    "prefill_8192": ("moe", 8192, 2),
                    # the 40-layer stack (26.4 GB of experts resident), each block's l_out the next block's input
-                   "stack40_b32": ("stack", 32, 40), "stack40_8192": ("stack", 8192, 40),
+                   "stack40_b3": ("stack", 3, 40), "stack40_b32": ("stack", 32, 40), "stack40_8192": ("stack", 8192, 40),
                    "dense_b1": ("dense", 1, 4), "dense_b8": ("dense", 8, 4), "dense_2048": ("dense", 2048, 2),
                    # the LM head (2048 -> 248 320, Q8_0: 540 MB per pass), two copies rotated
                    "lm_head_b1": ("lm_head", 1, 2), "lm_head_b3": ("lm_head", 3, 2), "lm_head_b8": ("lm_head", 8, 2)}
 
 
 def other_workload(args) -> int:
+    print(json.dumps(run_other(args, args.workload)))
+    return 0
+
+
+def run_other(args, workload) -> dict:
     """One of BASELINE's other configurations: the whole block, eager launches, HIP events on the launch
     stream over rotated layers.  One JSON line in the headline's format; the roofline is the block's own
     (algorithmic bytes or flops of a pass over its duration), not one kernel's."""
@@ -391,11 +417,11 @@ def other_workload(args) -> int:
     import llmxabe_amd as X
 
     torch.cuda.set_device(0)
-    kind, T, L = OTHER_WORKLOADS[args.workload]
+    kind, T, L = OTHER_WORKLOADS[workload]
     if kind == "lm_head":
         return lm_head_workload(args, T, L)
     if kind == "stack":
-        return stack_workload(args, T, L)
+        return stack_workload(args, workload, T, L)
     if kind == "moe":
         g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
         layers = [make_layer_device_only(X, g, seed=10_000 + 100 * l) for l in range(L)]
@@ -420,14 +446,14 @@ def other_workload(args) -> int:
             dst.copy_(src)
         del src, dst
     extra = {}
-    if args.workload == "prefill_512":
+    if workload == "prefill_512":
         # the skewed configuration: a seeded Zipf(s = 1.1) bias over the experts, added to the router logits before
         # routing (b_e = -s ln(rank_e) over a seeded permutation of the experts, i.e. selection odds proportional to rank^-1.1)
         extra["logit_bias"] = torch.from_numpy(X.zipf_logit_bias(256)).cuda()
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()
     reps_w = max(1, min(args.warmup, 64) // L)
-    reps = max(1, min(args.steps, 64 if T >= 512 else 320) // L)
+    reps = max(1, min(max(args.steps, 64), 64 if T >= 512 else 320) // L)   # (never fewer than 64 block passes)
     with torch.cuda.stream(stream):
         for _ in range(reps_w):
             for i in range(L):
@@ -447,7 +473,7 @@ def other_workload(args) -> int:
         distinct = len(np.unique(ids))
         byts = distinct * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES + 16384 + T * 2048 * 4 * 3
         flops = T * 57671680
-        cfg = {"workload": "moe_block_" + args.workload, "tokens": T, "num_experts": 256, "top_k": 8, "hidden": 2048,
+        cfg = {"workload": "moe_block_" + workload, "tokens": T, "num_experts": 256, "top_k": 8, "hidden": 2048,
                "intermediate": 512, "expert_quant": "Q6_K", "shared_and_router_quant": "Q8_0", "layers_rotated": L,
                "launch": "eager", "distinct_experts": distinct,
                "router_bias": "zipf s=1.1 (b_e = -1.1 ln rank_e), seed 5" if extra else None}
@@ -457,27 +483,30 @@ def other_workload(args) -> int:
     else:
         byts = 3 * 5120 * 17408 // 256 * 210
         flops = T * 3 * 2 * 5120 * 17408
-        cfg = {"workload": "dense_ffn_" + args.workload, "tokens": T, "hidden": 5120, "intermediate": 17408,
+        cfg = {"workload": "dense_ffn_" + workload, "tokens": T, "hidden": 5120, "intermediate": 17408,
                "quant": "Q6_K", "layers_rotated": L, "launch": "eager"}
     gbps, tflops = byts / (ms * 1e-3) / 1e9, flops / (ms * 1e-3) / 1e12
-    mfma_bound = args.workload in ("prefill_8192", "dense_2048")
+    mfma_bound = workload in ("prefill_8192", "dense_2048")
     roof = ({"kernel": "whole block", "bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
              "frac": tflops / MFMA_PEAK_TFLOPS, "traffic": None} if mfma_bound else
             {"kernel": "whole block", "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
              "frac": gbps / HBM_PEAK_GBPS, "traffic": None})
-    print(json.dumps({
+    del blk, layers, x, ffn_out, l_out
+    torch.cuda.empty_cache()
+    return {
         "metric": "MoE-block tokens/s at 1 GPU; decode HBM GB/s %peak; prefill MFMA util %", "value": T / (ms * 1e-3),
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": reps_w * L, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if T >= 64 else "f32",
         "data": "synthetic", "config": cfg, "roofline": roof, "algorithmic_bytes_per_step": byts, "flops_per_step": flops,
-        "cpu_baseline": None}))
-    return 0
+        "cpu_baseline": None}
 
 
-def stack_workload(args, T, L) -> int:
+def stack_workload(args, workload, T, L) -> dict:
     """L independently seeded MoE layers resident at once, one pass of T tokens through all of them per step:
-    layer l's l_out (residual + block output; the RMSNorm is the next block's first step) is layer l + 1's
-    input.  Ping-pong activation buffers, eager launches, HIP events on the launch stream."""
+    layer l's l_out (residual + block output) is layer l + 1's input, with the RMSNorm between them either as the
+    next block's first step (`value`: the reference-shaped calls) or folded into the launch that finishes l_out (the
+    `seam` object: xabe_moe_block_forward_seam, same bits).  Ping-pong activation buffers, eager launches, HIP events on
+    the launch stream."""
     import numpy as np
     import torch
 
@@ -493,27 +522,36 @@ def stack_workload(args, T, L) -> int:
     torch.cuda.synchronize()
     stream = torch.cuda.Stream()
 
-    def one_pass():
+    def one_pass(seam=False):
         cur = x0
         for i, w in enumerate(layers):
             nxt = bufs[i & 1]
-            blk.forward(w, cur, T, ffn_out, nxt)
+            if seam:  # one handle serves every layer: the tail writes the block's own normalised rows
+                blk.forward_seam(w, cur, T, None, nxt, input_normed=i > 0, skip_readback=True,
+                                 next_norm_weight=layers[i + 1].post_norm if i + 1 < L else None)
+            else:
+                blk.forward(w, cur, T, ffn_out, nxt)
             cur = nxt
         return cur
 
-    reps_w, reps = max(1, min(args.warmup, 4)), max(1, min(args.steps, 16 if T < 512 else 4))
+    reps_w, reps = max(1, min(args.warmup, 4)), max(2, min(args.steps, 16 if T < 512 else 4))
+    times, outs = {}, {}
     with torch.cuda.stream(stream):
-        for _ in range(reps_w):
-            one_pass()
-        stream.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for _ in range(reps):
-            out = one_pass()
-        e1.record(stream)
-        e1.synchronize()
-    ms = e0.elapsed_time(e1) / reps
-    finite = bool(torch.isfinite(out).all().item())
+        for seam in (False, True):
+            for _ in range(reps_w):
+                one_pass(seam)
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                out = one_pass(seam)
+            e1.record(stream)
+            e1.synchronize()
+            times[seam] = e0.elapsed_time(e1) / reps
+            outs[seam] = out.clone()
+    ms = times[False]
+    finite = bool(torch.isfinite(outs[False]).all().item())
+    same_bits = bool(torch.equal(outs[False].view(torch.int32), outs[True].view(torch.int32)))
     flops = L * T * 57671680
     weight_bytes = L * (256 * 3 * EXPERT_MATRIX_BYTES + SHARED_BYTES + ROUTER_BYTES)
     tflops = flops / (ms * 1e-3) / 1e12
@@ -530,19 +568,25 @@ def stack_workload(args, T, L) -> int:
              "frac": tflops / MFMA_PEAK_TFLOPS, "traffic": None} if mfma else
             {"kernel": "whole stack", "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
              "frac": gbps / HBM_PEAK_GBPS, "traffic": None})
-    print(json.dumps({
+    seam_ms = times[True]
+    del blk, layers, bufs, ffn_out, outs
+    torch.cuda.empty_cache()
+    return {
         "metric": "MoE-block tokens/s at 1 GPU; decode HBM GB/s %peak; prefill MFMA util %", "value": T / (ms * 1e-3),
         "unit": "tokens/s", "n_gpus": 1, "steps": reps, "warmup": reps_w, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if mfma else "f32", "data": "synthetic",
-        "config": {"workload": "moe_stack_" + args.workload, "layers": L, "tokens": T, "num_experts": 256, "top_k": 8,
+        "config": {"workload": "moe_stack_" + workload, "layers": L, "tokens": T, "num_experts": 256, "top_k": 8,
                    "hidden": 2048, "intermediate": 512, "expert_quant": "Q6_K", "shared_and_router_quant": "Q8_0",
                    "resident_weight_bytes": weight_bytes, "launch": "eager", "us_per_layer": ms * 1e3 / L,
                    "output_finite": finite},
-        "roofline": roof, "algorithmic_bytes_per_step": byts, "flops_per_step": flops, "cpu_baseline": None}))
-    return 0
+        "seam": {"what": "the same pass with every layer boundary's RMSNorm folded into the launch that finishes l_out "
+                         "(xabe_moe_block_forward_seam; no ffn_out / routed read-back tensors)",
+                 "ms_per_step": seam_ms, "us_per_layer": seam_ms * 1e3 / L, "tokens_per_s": T / (seam_ms * 1e-3),
+                 "speedup": ms / seam_ms, "same_bits_as_unfused": same_bits},
+        "roofline": roof, "algorithmic_bytes_per_step": byts, "flops_per_step": flops, "cpu_baseline": None}
 
 
-def lm_head_workload(args, T, L) -> int:
+def lm_head_workload(args, T, L) -> dict:
     """The LM-head GEMV over the real head's shape (Q8_0), logits for T tokens per step; HIP events on the
     launch stream; the CPU leg is the oracle's sequential gemv over a slice of the vocabulary."""
     import time
@@ -592,16 +636,15 @@ def lm_head_workload(args, T, L) -> int:
         dt = time.perf_counter() - t0
         cpu = {"value": n * rows / g.vocab / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
                "sample": f"sequential gemv over {rows} of the 248320 rows (dequantised beforehand), {n} token passes, scaled to the whole vocabulary"}
-    print(json.dumps({
+    return ({
         "metric": "LM-head tokens/s at 1 GPU; HBM GB/s %peak", "value": T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
         "steps": steps, "warmup": reps_w * L, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": args.workload, "tokens": T, "hidden": g.hidden, "vocab": g.vocab, "format": "Q8_0",
+        "config": {"workload": "lm_head_b%d" % T, "tokens": T, "hidden": g.hidden, "vocab": g.vocab, "format": "Q8_0",
                    "weight_passes": g.weight_passes(T), "heads_rotated": L, "launch": "eager"},
         "roofline": {"kernel": "k_lm_head_quant", "bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": gbps / HBM_PEAK_GBPS, "traffic": None},
-        "algorithmic_bytes_per_step": byts, "cpu_baseline": cpu}))
-    return 0
+        "algorithmic_bytes_per_step": byts, "cpu_baseline": cpu})
 
 
 def make_layer_device_only(X, g, seed):
@@ -644,9 +687,9 @@ def cpu_baseline(w, g, x, T, budget_s):
                 return n, el, deq, mv
 
     n1, el1, deq1, mv1 = run(1, budget_s * 0.7)
-    cores = min(oracle.num_threads(), 16)
+    cores = min(oracle.num_threads(), 16)   # the box's CPU share for one GPU is 16 cores, whatever nproc shows
     nt, elt, _, _ = run(cores, budget_s * 0.3)
-    return {"value": T * n1 / el1, "unit": "tokens/s", "cores": 1, "kind": "port",
+    return {"value": T * n1 / el1, "unit": "tokens/s", "cores": 1, "kind": "port", "host_nproc": os.cpu_count(),
             "sample": f"{n1} passes of the same {T}-token block on layer 0 (dequantise selected experts + sequential "
                       f"fp32 matvecs), {el1:.1f} s; dequant {deq1 / n1 * 1e3:.0f} ms + matvec {mv1 / n1 * 1e3:.0f} ms per pass",
             "openmp": {"value": T * nt / elt, "cores": cores, "passes": nt, "seconds": elt}}

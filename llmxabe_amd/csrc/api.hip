@@ -521,7 +521,8 @@ static int alloc_buffers(const xabe_moe_kernels* k, void* stream, int scope, boo
                             : 0;
   A(&b->router_partial, b->n_router_partial);
   // decode widths: one arrival counter per token for the seam's tail in the third launch (decode_block.hip)
-  A(&b->seam_arrivals, (routed && g.max_tokens <= 32) ? g.max_tokens : 0);
+  b->n_seam_arrivals = (routed && g.max_tokens <= 32) ? g.max_tokens * seam_counter_ints_per_token() : 0;
+  A(&b->seam_arrivals, b->n_seam_arrivals);
   b->bytes = total;
   b->valid_published = 0;
   if (st != XABE_OK) {

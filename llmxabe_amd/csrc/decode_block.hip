@@ -56,6 +56,8 @@ constexpr int kPreRouteMinTokens = 8;
 // 32 tokens with one pair at a time, 135 us two at a time (sharing the dequantisation takes ~230 registers); the
 // pairs of an expert run one after the other there, and a third of the workgroups find no pair at all.)
 constexpr int kXcdGroupMinTokens = 24;
+// the seam's arrival counters: per token one counter and one per group of kSeamGroup workgroups, 128 bytes apart
+constexpr int kSeamGroup = 16, kSeamMaxGroups = 64, kSeamCountersPerToken = 1 + kSeamMaxGroups, kSeamCounterStride = 32;
 constexpr int kMaxTopK = 8;       // contributions held in registers by k_decode_down
 constexpr int kMaxInter = 512;    // intermediate width staged in LDS by k_decode_down
 // Steps per wavefront of the first launch: a wavefront reads 24 KB of activation rows and norm weights for the 2-4 KB
@@ -473,6 +475,8 @@ __global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
   __shared__ __attribute__((aligned(16))) float s_x[(kMaxTopK + 1) * kMaxInter];
   __shared__ float s_xs[(kMaxTopK + 1) * kMaxInter / 8];  // -32 * (sum of each run of eight), Q6_K's code offset
   __shared__ float s_part[RS][kHalf][RPS];               // the second wavefront's weighted row sums
+  __shared__ int s_arrived;                              // the seam's tail: storing wavefronts of this workgroup that are done
+  if (threadIdx.x == 0) s_arrived = 0;                   // (two barriers before anyone counts)
   int t = blockIdx.x / a.tiles_d, tile = blockIdx.x % a.tiles_d;
   if (a.max_tokens >= kXcdGroupMinTokens && (a.tiles_d & 7) == 0) {
     // wide batches (see kXcdGroupMinTokens): all tokens of one row tile next to each other on one XCD
@@ -612,21 +616,33 @@ __global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
   XABE_TRACE(2, 3);
   if (!a.next_normed) return;
   // The seam (docs/BENCHMARKS.md:1376 of the reference: the next layer's RMSNorm in the combine's tail).  A token's
-  // row is finished by tiles_d workgroups; each counts its arrival once its stores have been acknowledged, and the
-  // one that arrives last reads the row back (agent-scope loads: the other workgroups' stores went through to memory,
-  // no fence, whose L2 write-back costs microseconds here), forms the RMS scale in the canonical order and writes
-  // the normalised row: the bits of the stand-alone RMSNorm launch on l_out.
-  __shared__ int s_last;
+  // row is finished by tiles_d workgroups, and the wavefront that finishes it last applies the norm.  Arrivals are
+  // counted in three levels so that no counter sees more than a few dozen of them (atomics on one address are served
+  // one after the other, ~70 ns each: 256 arrivals on one counter cost 18 us per pass at 32 tokens): the storing
+  // wavefronts of a workgroup in LDS, 16 workgroups on a group counter, the groups on the token's counter, every
+  // counter on a 128-byte line of its own.  A wavefront counts itself once its own stores are acknowledged (they go
+  // through to memory: no fence, whose L2 write-back costs microseconds here), so whoever sees a count complete knows
+  // all stores below it have landed.  No workgroup barrier: the other wavefronts are done.
+  if (second) return;
   __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  if (threadIdx.x == 0)
-    s_last = __hip_atomic_fetch_add(a.arrivals + t, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.tiles_d - 1;
-  __syncthreads();
-  if (!s_last || wave != 0) return;
-  if (lane == 0) __hip_atomic_store(a.arrivals + t, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next pass
+  int prev = 0;
+  if (lane == 0) prev = __hip_atomic_fetch_add(&s_arrived, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  if (__builtin_amdgcn_readfirstlane(prev) != RS - 1) return;
+  int* const token_ctr = a.arrivals + (size_t)t * kSeamCountersPerToken * kSeamCounterStride;
+  const int groups = (a.tiles_d + kSeamGroup - 1) / kSeamGroup, grp = tile / kSeamGroup;
+  const int in_group = min(kSeamGroup, a.tiles_d - grp * kSeamGroup);
+  int* const group_ctr = token_ctr + (1 + grp) * kSeamCounterStride;
+  if (lane == 0) prev = __hip_atomic_fetch_add(group_ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (__builtin_amdgcn_readfirstlane(prev) != in_group - 1) return;
+  if (lane == 0) {
+    __hip_atomic_store(group_ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (zero again for the next pass)
+    prev = __hip_atomic_fetch_add(token_ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (__builtin_amdgcn_readfirstlane(prev) != groups - 1) return;
+  if (lane == 0) __hip_atomic_store(token_ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   // the row comes in coalesced (element 64 j + lane per load) and changes hands through LDS (s_x is free now), padded
   // by four floats per 32 as the first launch pads its rows
-  float* s_l = s_x;
+  float* s_l = s_x;  // (free since the last barrier; one wavefront per workgroup at most gets here: a workgroup serves one token)
   const float* lrow = a.l_out + (size_t)t * a.H;
   float in[32];
 #pragma unroll
@@ -722,6 +738,8 @@ static bool launch_shape(const Launch& l, int gq, int dq, int sgq, int sdq, int 
   return false;
 }
 
+size_t seam_counter_ints_per_token() { return (size_t)kSeamCountersPerToken * kSeamCounterStride; }
+
 bool decode_block_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, const xabe_moe_layer_weights* w) {
   const xabe_moe_geometry& g = k->g;
   if (g.max_tokens > kDecodeBlockMaxTokens || k->force_community || b->scope != XABE_SCOPE_ROUTED) return false;
@@ -742,7 +760,7 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
   DecodeArgs a;
   memset(&a, 0, sizeof(a));
   if (seam && seam->next_normed) {
-    if (!b->seam_arrivals)
+    if (!b->seam_arrivals || b->n_seam_arrivals < g.max_tokens * seam_counter_ints_per_token())
       return set_error(XABE_ERR_INVALID_ARGUMENT, "decode block: these buffers carry no arrival counters for the seam");
     a.next_w = seam->next_w;
     a.next_normed = seam->next_normed;

@@ -77,6 +77,7 @@ int check_layer_stacks(const xabe_moe_kernels* k, const xabe_moe_layer_weights* 
 // The seam between this block and the next as the decode launches see it: `input_normed`: `normed` holds the pass's
 // rows already; `next_normed` (null: the pass ends at l_out): where the third launch's last workgroup per token
 // writes rms_norm(l_out, next_w, next_eps), `next_normed_h` (may be null) its fp16 copy.
+size_t seam_counter_ints_per_token();  // ints of arrival counters the seam's tail needs per token (decode_block.hip)
 struct DecodeSeam {
   bool input_normed;
   const float* next_w;
@@ -187,7 +188,8 @@ struct xabe_moe_buffers {
   // rewrites the device lists without touching the fields above, so from then on only a forward inside a capture
   // that holds its own build trusts them; eager forwards always make their own
   bool tiles_graph_owned;
-  int32_t* seam_arrivals;  // [max_tokens], decode widths: arrival counters of the seam's tail (zero between passes)
+  int32_t* seam_arrivals;  // decode widths: arrival counters of the seam's tail (zero between passes)
+  size_t n_seam_arrivals;
   float* router_partial;  // [split][token][expert]: the router GEMM's contraction splits at mid widths
   size_t n_router_partial;
   size_t bytes;
