@@ -116,6 +116,9 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the two prefill legs of the headline run")
     ap.add_argument("--no-calibration", action="store_true", help="skip the read / matrix-instruction calibration legs")
+    ap.add_argument("--mfma-form", type=int, default=0, choices=[0, 1, 2],
+                    help="--workload prefill_*: which grouped-GEMM kernel the routed launches take (2: the "
+                         "specialised-wavefront form, same bits, kept for comparison)")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the compact legs of BASELINE's other configurations (decode batch 32, the dense sibling, the 40-layer stack)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -426,6 +429,7 @@ def run_other(args, workload) -> dict:
         g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
         layers = [make_layer_device_only(X, g, seed=10_000 + 100 * l) for l in range(L)]
         blk = X.MoeBlock(g)
+        blk.set_mfma_form(getattr(args, "mfma_form", 0))
         blk.publish_tokens(T)
         width = 2048
     else:

@@ -138,6 +138,12 @@ int xabe_moe_kernels_tensor_cores_enabled(const xabe_moe_kernels* k);           
 /* M:5432-5434: no community-format kernels exist here; `on != 0` is accepted and recorded only. */
 int xabe_moe_kernels_force_community(xabe_moe_kernels* k, int on);
 /* M:5450-5452: pin the fp32 decode kernels at any width so rows equal plain decode bit for bit. */
+/* No counterpart in the reference (a test and comparison switch like force_community): which of the two
+ * matrix-core grouped-GEMM kernels the routed launches of a wide pass take.  0 (default) and 1: the kernel whose
+ * wavefronts all load, dequantise and multiply in turn; 2: the kernel whose wavefronts are specialised (half of them
+ * multiply, half dequantise) wherever the shape allows: same bits, measured slower at every width, kept as the
+ * reproducible record of that comparison. */
+int xabe_moe_kernels_set_mfma_form(xabe_moe_kernels* k, int form);
 int xabe_moe_kernels_set_exact_decode_regime(xabe_moe_kernels* k, int on);
 
 /* MoeKernels::buffers (M:5338-5340) / shared_only_buffers (M:5354-5360) */
@@ -307,6 +313,7 @@ int xabe_moe_block_set_exact_decode_regime(xabe_moe_block* blk, int on); /* B:10
  * combine) that compute the same values bit for bit.  `on` = 0 keeps one launch per step as the reference
  * has them (B:1091-1329); the switch exists for tests and measurement. */
 int xabe_moe_block_set_fused_decode(xabe_moe_block* blk, int on);
+int xabe_moe_block_set_mfma_form(xabe_moe_block* blk, int form); /* xabe_moe_kernels_set_mfma_form on the block's kernels */
 /* Measurement hook, no counterpart in the reference: ONE of the three decode launches (0: logits + shared
  * gate/up, 1: route + gate/up, 2: down + combine) with the arguments of xabe_moe_block_forward, so that a
  * launch can be timed and profiled alone.  Stage n reads what stages < n of an earlier call left in the

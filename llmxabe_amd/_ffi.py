@@ -86,6 +86,7 @@ _SIGNATURES = {
     "xabe_moe_kernels_tensor_cores_enabled": (C.c_int, [vp]),
     "xabe_moe_kernels_force_community": (C.c_int, [vp, C.c_int]),
     "xabe_moe_kernels_set_exact_decode_regime": (C.c_int, [vp, C.c_int]),
+    "xabe_moe_kernels_set_mfma_form": (C.c_int, [vp, C.c_int]),
     "xabe_moe_buffers_new": (C.c_int, [vp, vp, C.POINTER(vp)]),
     "xabe_moe_shared_only_buffers_new": (C.c_int, [vp, vp, C.c_int, C.POINTER(vp)]),
     "xabe_moe_buffers_free": (None, [vp]),
@@ -130,6 +131,7 @@ _SIGNATURES = {
     "xabe_moe_block_disable_tensor_cores": (C.c_int, [vp]),
     "xabe_moe_block_set_exact_decode_regime": (C.c_int, [vp, C.c_int]),
     "xabe_moe_block_set_fused_decode": (C.c_int, [vp, C.c_int]),
+    "xabe_moe_block_set_mfma_form": (C.c_int, [vp, C.c_int]),
     "xabe_moe_block_forward_stage": (C.c_int, [vp, vp, vp, vp, sz, vp, vp, sz, vp, sz, C.c_int]),
     "xabe_moe_block_tensor_cores_enabled": (C.c_int, [vp]),
     "xabe_moe_block_normed": (vp, [vp, C.POINTER(sz)]),

@@ -63,6 +63,7 @@ class MoeBlock:
     def set_exact_decode_regime(self, on: bool): check(_ffi.lib().xabe_moe_block_set_exact_decode_regime(self._h, int(on)))
     def tensor_cores_enabled(self) -> bool: return bool(_ffi.lib().xabe_moe_block_tensor_cores_enabled(self._h))
     def set_fused_decode(self, on: bool): check(_ffi.lib().xabe_moe_block_set_fused_decode(self._h, int(on)))
+    def set_mfma_form(self, form: int): check(_ffi.lib().xabe_moe_block_set_mfma_form(self._h, form))
 
     def publish_tokens(self, tokens: int):
         check(_ffi.lib().xabe_moe_block_publish_tokens(self._h, _stream(), tokens))

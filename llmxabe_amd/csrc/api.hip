@@ -454,6 +454,12 @@ int xabe_moe_kernels_force_community(xabe_moe_kernels* k, int on) {
   k->force_community = on != 0;
   return XABE_OK;
 }
+int xabe_moe_kernels_set_mfma_form(xabe_moe_kernels* k, int form) {
+  if (!k) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_mfma_form: null handle");
+  if (form < 0 || form > 2) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_mfma_form: form %d is not 0 (by width), 1 or 2", form);
+  k->mfma_form = form;
+  return XABE_OK;
+}
 int xabe_moe_kernels_set_exact_decode_regime(xabe_moe_kernels* k, int on) {
   if (!k) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_exact_decode_regime: null handle");
   k->exact_regime = on != 0;

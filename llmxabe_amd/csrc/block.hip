@@ -260,6 +260,10 @@ int xabe_moe_block_set_exact_decode_regime(xabe_moe_block* blk, int on) {
   if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_exact_decode_regime: null handle");
   return xabe_moe_kernels_set_exact_decode_regime(blk->moe, on);
 }
+int xabe_moe_block_set_mfma_form(xabe_moe_block* blk, int form) {
+  if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_mfma_form: null handle");
+  return xabe_moe_kernels_set_mfma_form(blk->moe, form);
+}
 int xabe_moe_block_set_fused_decode(xabe_moe_block* blk, int on) {
   if (!blk) return set_error(XABE_ERR_INVALID_ARGUMENT, "set_fused_decode: null handle");
   blk->fused_decode = on != 0;

@@ -147,6 +147,7 @@ struct xabe_moe_kernels {
   bool tensor_cores;
   bool exact_regime;
   bool force_community;
+  int mfma_form;  // matrix-core regime, routed launches: 0 chosen by width, 1 k_mfma_expert, 2 k_mfma_pc (mfma.hip)
   int device;
   int num_cus;
 };

@@ -624,6 +624,404 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_m
   }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// The same grouped GEMM with the wavefronts of a workgroup specialised: an alternative form of the routed launches,
+// selected with xabe_moe_kernels_set_mfma_form(k, 2).  Same bits as k_mfma_expert; measured within 0-7 % of it and
+// never ahead (8192 tokens: gate/up 461 against 421 us, down 333 against 308), so it is not the default.  It is kept
+// because it is the measured answer to "would wavefronts that only dequantise beside wavefronts that only multiply
+// overlap the two kinds of work": they do not.  On a SIMD the producers' vector instructions and the consumers'
+// matrix instructions take turns (per 64-element step and SIMD: 1024 cycles of matrix instructions + 1144 of vector
+// instructions of work, 1320 ns = 3170 cycles of wall time; either kind alone, the other removed, still takes ~2600),
+// so what decides the time is the sum of the two per token row, and that sum is smallest for the tallest token tile
+// (one dequantisation per expert), whose accumulators only fit a few fat wavefronts: k_mfma_expert's 384-row form.
+//
+// A workgroup is sixteen wavefronts with two jobs:
+//   consumers (wavefronts 0-7, 2 row halves x 4 column quarters): request the activation tile three steps ahead
+//     (global memory -> LDS, no registers) and multiply THIS step's tiles: 64 token rows x 64 weight rows each;
+//   producers (wavefronts 8-15): keep the raw weight bytes of the next two 128-element blocks of the contraction in
+//     flight and dequantise the next step's weight tile into LDS.
+// A step is 64 contraction elements; the weight tile is double-buffered and the activation tile sits in a ring of
+// four, so there is ONE barrier per step and nobody waits inside a step for memory it has just asked for: a
+// consumer's pieces were requested three steps earlier, a producer's raw bytes two to four steps earlier, and each
+// kind of wavefront counts only its own loads (the wait counters are per wavefront).
+//
+// The tile is 128 token rows x 256 weight rows (gate/up: 128 + 128): twice k_mfma_expert's weight rows per
+// activation byte (with 128 weight rows and a one-step-ahead activation tile the consumers waited for L2 every step:
+// 623 us).
+// Per output element the operands and the order of the matrix instructions are k_mfma_expert's (ascending
+// contraction index, 16 elements per instruction), so the bits are the same.
+// A Q6_K unit (32 codes of one row: 8 at each of four places 32 elements apart) spans two steps: its raw registers
+// are loaded once per 128-element block and dequantised a half at a time.
+// LDS: rows of 64 halfs (128 bytes: two rows to a 256-byte line of the 64 banks), 16-byte chunks XOR-swizzled by
+// pc_swizzle(row) in both tiles.  Fragment reads are served sixteen lanes at a time (sixteen rows, one chunk each): the
+// eight rows of either parity must put the chunk at eight different positions, hence a permutation of (row >> 1) & 7;
+// the dequantised stores (lanes = rows x the four chunks 4 jj .. 4 jj + 3) need rows two apart to differ in the
+// position's high bit, hence the bit order.  (With row & 7 the bank-conflict counter showed every fragment read taking
+// twice its cycles.)
+constexpr int kPK = 64;        // contraction elements per step
+constexpr int kPM = 128;       // token rows per tile
+constexpr int kPR = 256;       // weight rows per tile
+constexpr int kPARing = 4;     // activation tiles in LDS
+constexpr int kPAhead = 3;     // steps between an activation tile's request and its use
+constexpr int kPCWaves = 8;    // consumer wavefronts (as many producers)
+constexpr int kPAInstr = kPM / (8 * kPCWaves);  // activation-piece instructions per consumer wavefront and step (1 KB = 8 rows each)
+
+__device__ __forceinline__ int pc_swizzle(int row) { return (((row >> 1) & 1) << 2) | ((row >> 2) & 3); }
+
+constexpr size_t mfma_pc_lds_bytes() {
+  return (size_t)kPARing * kPM * kPK * sizeof(_Float16) + (size_t)2 * kPR * kPK * sizeof(_Float16) + (size_t)2 * 3 * kPM * sizeof(int);
+}
+
+// half HH (codes at places 2 HH and 2 HH + 1) of a Q6_K unit -> chunks (jj * 4 + l8) of the row's 64-element tile row
+template <int HH>
+__device__ __forceinline__ void q6_half_unit_to_lds(const Q6Pend& r, int l8, _Float16* brow, int swz) {
+  const int is8 = (l8 >> 1) * 8;
+  const uint32_t sw = (HH ? r.sc.y : r.sc.x) >> is8;
+  const float d = f16_bits_to_f32(r.dh) * kWScale;
+  const float ds[2] = {d * (float)(int8_t)(sw & 0xff), d * (float)(int8_t)((sw >> 16) & 0xff)};
+  uint32_t c[2][2];
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    const uint32_t a = w ? r.qa.y : r.qa.x, b = w ? r.qb.y : r.qb.x, h = w ? r.qh.y : r.qh.x;
+    if (HH == 0) {
+      c[w][0] = (a & 0x0F0F0F0Fu) | ((h << 4) & 0x30303030u);
+      c[w][1] = (b & 0x0F0F0F0Fu) | ((h << 2) & 0x30303030u);
+    } else {
+      c[w][0] = ((a >> 4) & 0x0F0F0F0Fu) | (h & 0x30303030u);
+      c[w][1] = ((b >> 4) & 0x0F0F0F0Fu) | ((h >> 2) & 0x30303030u);
+    }
+  }
+  const half2v off = {(_Float16)-1056.0f, (_Float16)-1056.0f};  // 1024 (perm bias) + 32 (code centre)
+#pragma unroll
+  for (int jj = 0; jj < 2; ++jj) {
+    const _Float16 sh = (_Float16)ds[jj];
+    const half2v s = {sh, sh};
+    *reinterpret_cast<u32x4*>(brow + ((jj * 4 + l8) ^ swz) * 8) = pack8(c[0][jj], c[1][jj], off, s);
+  }
+}
+// a Q8_0 block -> chunks 4 blk .. 4 blk + 3 of the row's 64-element tile row
+__device__ __forceinline__ void q8_block_to_lds(const Q8Pend& r, int blk, _Float16* brow, int swz) {
+  const _Float16 sh = (_Float16)(f16_bits_to_f32(r.dh) * kWScale);
+  const half2v s = {sh, sh};
+  const half2v off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+  const uint32_t q[8] = {r.lo[0], r.lo[1], r.lo[2], r.lo[3], r.hi[0], r.hi[1], r.hi[2], r.hi[3]};
+#pragma unroll
+  for (int w = 0; w < 4; ++w)
+    *reinterpret_cast<u32x4*>(brow + ((blk * 4 + w) ^ swz) * 8) = pack8(q[2 * w] ^ 0x80808080u, q[2 * w + 1] ^ 0x80808080u, off, s);
+}
+
+template <int QUANT, int NM>
+__global__ void __launch_bounds__(1024, 4) k_mfma_pc(MfmaArgs a) {
+  constexpr int kTable = 3 * kPM;
+  extern __shared__ __attribute__((aligned(16))) uint8_t mfma_smem[];
+  _Float16* sA = reinterpret_cast<_Float16*>(mfma_smem);          // [kPARing][128][64]
+  _Float16* sB = sA + kPARing * kPM * kPK;                        // [2][256][64]
+  int* sArow = reinterpret_cast<int*>(sB + 2 * kPR * kPK);        // [2][3 x 128]: activation row, output row (-1: dead), scale
+  int* sOrow = sArow + kPM;
+  float* sScale = reinterpret_cast<float*>(sOrow + kPM);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool producer = wave >= kPCWaves;
+  const int n_ntiles = a.n_rows / (NM == 2 ? kPR / 2 : kPR);
+  const int n_mtiles = a.tile_list[0];
+  const int total = n_mtiles * n_ntiles;
+  const int nks = a.K / kPK;  // a multiple of four (whole superblocks), at least eight (checked by the host)
+  const size_t row_bytes = QUANT == kQ6K ? (size_t)(a.K / 256) * kQ6KBytes : (size_t)(a.K / 32) * kQ8Bytes;
+
+  // which items this workgroup takes: k_mfma_expert's dealing (an XCD walks a contiguous eighth of the token tiles)
+  const bool by_xcd = (gridDim.x & 7u) == 0 && total >= 2 * (int)gridDim.x && n_mtiles >= 8;
+  const int xcd = blockIdx.x & 7;
+  const int m_lo = by_xcd ? (int)((long long)n_mtiles * xcd / 8) : 0;
+  const int m_hi = by_xcd ? (int)((long long)n_mtiles * (xcd + 1) / 8) : n_mtiles;
+  const int first = by_xcd ? (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  const int stride = by_xcd ? (int)(gridDim.x >> 3) : (int)gridDim.x;
+  const int local_total = (m_hi - m_lo) * n_ntiles;
+  if (first >= local_total) return;
+  const int n_items = (local_total - first + stride - 1) / stride;
+  const int n_steps = n_items * nks;  // a multiple of four
+
+  struct Item { int e, m0, rows, nt; };
+  auto decode = [&](int item) __attribute__((always_inline)) {
+    const int mt = m_lo + item / n_ntiles;
+    typedef int int4v __attribute__((ext_vector_type(4)));
+    int4v ent;
+    const int* p = a.tile_list + 4 + 4 * mt;
+    asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ent) : "s"(p));
+    return Item{ent.x, ent.y, ent.z, item % n_ntiles};
+  };
+
+  // ---- the first item's row tables, by the consumers' threads; everyone meets at one barrier before the steps
+  if (tid < kPM) {
+    const Item it = decode(first);
+    int arow = 0, orow = -1;
+    float sc = 1.0f;
+    if (tid < it.rows) {
+      const int slot = it.m0 + tid, flat = a.sorted_token_ids[slot];
+      if (NM == 2) { arow = flat / a.top_k; orow = slot; }
+      else { arow = slot; orow = flat; sc = a.topk_weights[flat]; }
+    }
+    sArow[tid] = arow;
+    sOrow[tid] = orow;
+    sScale[tid] = sc;
+  }
+  __syncthreads();
+
+  if (producer) {
+    // ================================================================= producers
+    const int ptid = tid - 64 * kPCWaves;
+    // Q6_K: units (row rb0 + 128 i, place l8) of the 256-row tile, two per thread, raw registers per 128-element block
+    // Q8_0: one 34-byte block per thread and step: row q8row, block q8blk of the step's two
+    constexpr int kUnits = QUANT == kQ6K ? 2 : 1;
+    const int du = ptid & 3, rb0 = ptid >> 2;
+    const int q8row = ptid & 255, q8blk = ptid >> 8;
+    const ptrdiff_t up_minus_gate = NM == 2 ? a.w1 - a.w0 : 0;
+    const uint8_t* wrow[kUnits];
+    auto tile_row = [&](int i) __attribute__((always_inline)) { return QUANT == kQ6K ? rb0 + 128 * i : q8row; };
+    auto set_wrow = [&](const Item& it) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < kUnits; ++i) {
+        const int rb = tile_row(i);
+        const uint8_t* base = a.w0;
+        int wr;
+        if (NM == 2) {
+          // tile rows in groups of 32: gate columns, the matching up columns, the next 32 gate columns, ...
+          const int grp = rb >> 6, which = (rb >> 5) & 1, c = rb & 31;
+          base += which ? up_minus_gate : (ptrdiff_t)0;
+          wr = it.nt * (kPR / 2) + grp * 32 + c;
+        } else {
+          wr = it.nt * kPR + rb;
+        }
+        wrow[i] = base + (size_t)it.e * a.expert_bytes + (size_t)wr * row_bytes;
+      }
+    };
+    // raw bytes in flight: Q6_K two blocks of 128 (sets by block parity), Q8_0 four steps (sets by step & 3)
+    constexpr int kSets = QUANT == kQ6K ? 2 : 4;
+    typename std::conditional<QUANT == kQ6K, Q6Pend, Q8Pend>::type raw[kSets][kUnits];
+    // the load stream runs ahead of the dequantisation, across item boundaries: its own item counter and pointers
+    int ld_item = 0, ld_k = 0;  // next load: item index (0 .. n_items), and block (Q6_K) or step (Q8_0) within it
+    const int ld_per_item = QUANT == kQ6K ? nks / 2 : nks;
+    set_wrow(decode(first));
+    auto issue = [&](auto set_c) __attribute__((always_inline)) {
+      constexpr int S = decltype(set_c)::value;
+      // (past the last item the stream re-reads the last item's first blocks and drops them: every fill issues
+      // the same loads, so the compiler's count of what is in flight is exact on every path)
+#pragma unroll
+      for (int i = 0; i < kUnits; ++i) {
+        if constexpr (QUANT == kQ6K) {
+          // block ld_k covers superblock ld_k >> 1, half ld_k & 1
+          q6_issue(wrow[i] + (size_t)(ld_k >> 1) * kQ6KBytes, ld_k & 1, du, raw[S][i]);
+        } else {
+          q8_issue(wrow[i] + (size_t)(ld_k * 2 + q8blk) * kQ8Bytes, raw[S][i]);
+        }
+      }
+      if (++ld_k == ld_per_item) {
+        ld_k = 0;
+        if (++ld_item < n_items) set_wrow(decode(first + ld_item * stride));
+      }
+    };
+    // fill of the weight tile of global step T (T & 3 == P): into buffer T & 1
+    auto fill = [&](auto p_c) __attribute__((always_inline)) {
+      constexpr int P = decltype(p_c)::value;
+      _Float16* dst = sB + (P & 1) * kPR * kPK;
+      if constexpr (QUANT == kQ6K) {
+        constexpr int S = P >> 1, HH = P & 1;
+#pragma unroll
+        for (int i = 0; i < kUnits; ++i) {
+          const int rb = tile_row(i);
+          q6_half_unit_to_lds<HH>(raw[S][i], du, dst + rb * kPK, pc_swizzle(rb));
+        }
+        if constexpr (HH == 1) issue(std::integral_constant<int, S>{});  // the block after next, into the registers just released
+      } else {
+#pragma unroll
+        for (int i = 0; i < kUnits; ++i) {
+          const int rb = tile_row(i);
+          q8_block_to_lds(raw[P][i], q8blk, dst + rb * kPK, pc_swizzle(rb));
+        }
+        issue(std::integral_constant<int, P>{});
+      }
+    };
+    order_fence();
+    issue(std::integral_constant<int, 0>{});
+    order_fence();
+    issue(std::integral_constant<int, 1>{});
+    order_fence();
+    if constexpr (QUANT != kQ6K) {
+      issue(std::integral_constant<int, 2>{});
+      order_fence();
+      issue(std::integral_constant<int, 3>{});
+      order_fence();
+    }
+    fill(std::integral_constant<int, 0>{});
+    for (int T = 0; T < n_steps; T += 4) {
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      fill(std::integral_constant<int, 1>{});
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      fill(std::integral_constant<int, 2>{});
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      fill(std::integral_constant<int, 3>{});
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (T + 4 < n_steps) fill(std::integral_constant<int, 0>{});
+    }
+    return;
+  }
+
+  // ================================================================= consumers
+  const int wm = wave >> 2, wq = wave & 3;  // row half (blocks b % 2 == wm), column quarter (64 weight rows)
+  // piece q = i * kPCWaves + wave of the tile: rows 8 q .. 8 q + 7; lane: row 8 q + (lane >> 3), position lane & 7, which holds
+  // chunk (lane & 7) ^ pc_swizzle(row).  Every piece is requested, dead rows' too (from the tile's first row): the count of
+  // requests in flight is then the same at every step, which is what the waits below rely on.
+  uint32_t arow_off[kPAInstr], arow_nxt[kPAInstr];
+  auto set_arow = [&](int tb, uint32_t (&dst)[kPAInstr]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < kPAInstr; ++i) {
+      const int row = 8 * (i * kPCWaves + wave) + (lane >> 3), chunk = (lane & 7) ^ pc_swizzle(row);
+      dst[i] = (uint32_t)sArow[tb * kTable + row] * (uint32_t)a.K + (uint32_t)chunk * 8u;
+    }
+  };
+  const uint32_t lds_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)sA;
+  auto move_a = [&](int slot, int ks, const uint32_t (&off)[kPAInstr]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < kPAInstr; ++i) {
+      const int q = i * kPCWaves + wave;
+      const uint32_t voff = (off[i] + (uint32_t)ks * (uint32_t)kPK) * 2u;
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_a + (uint32_t)(slot * kPM * kPK * 2) + (uint32_t)q * 1024u);
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(a.a), "s"(dst) : "memory", "m0");
+#pragma clang diagnostic pop
+    }
+  };
+
+  Item cur = decode(first);
+  set_arow(0, arow_off);
+#pragma unroll
+  for (int i = 0; i < kPAInstr; ++i) arow_nxt[i] = arow_off[i];
+  // the first kPAhead tiles (an item has at least eight steps)
+#pragma unroll
+  for (int t = 0; t < kPAhead; ++t) move_a(t, t, arow_off);
+  int step = 0;
+  for (int idx = 0; idx < n_items; ++idx) {
+    const bool has_next = idx + 1 < n_items;
+    const Item nxt = has_next ? decode(first + (idx + 1) * stride) : cur;
+    asm volatile("" ::"s"(nxt.e), "s"(nxt.m0), "s"(nxt.rows), "s"(nxt.nt));
+    const int tb = idx & 1;
+    int n_flat = 0;
+    float n_sc = 1.0f;
+
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    // live 32-row blocks of this consumer row: block b = 2 mi + wm holds rows 32 b ..
+    const int nb = min(max((cur.rows - 32 * wm + 63) / 64, 0), 2);
+
+#pragma unroll 1
+    for (int ks = 0; ks < nks; ++ks, ++step) {
+      // this step's tiles are there: my own pieces of it (requested three steps ago; memory operations retire in
+      // order, so all but the two newer tiles' requests covers them) have landed, and past the barrier so have
+      // everyone else's and the producers' weight tile.  Near the end of the workgroup's work fewer requests follow.
+      order_fence();
+      if (step + kPAhead <= n_steps) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((kPAhead - 1) * kPAInstr) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      order_fence();
+      // the next item's row tables, in three parts spread over this item's steps so that nothing waits for a load
+      // it has just issued: flat selection index, output scale, the table itself
+      if (has_next && tid < kPM) {
+        if (ks == 0) n_flat = a.sorted_token_ids[nxt.m0 + min(tid, nxt.rows - 1)];
+        if (NM == 1 && ks == 2) n_sc = a.topk_weights[n_flat];
+        if (ks == nks - kPAhead - 2) {
+          int arow = 0, orow = -1;
+          if (tid < nxt.rows) {
+            const int slot = nxt.m0 + tid;
+            if (NM == 2) { arow = n_flat / a.top_k; orow = slot; }
+            else { arow = slot; orow = n_flat; }
+          }
+          sArow[(tb ^ 1) * kTable + tid] = arow;
+          sOrow[(tb ^ 1) * kTable + tid] = orow;
+          sScale[(tb ^ 1) * kTable + tid] = n_sc;
+        }
+      }
+      if (has_next && ks == nks - kPAhead - 1) set_arow(tb ^ 1, arow_nxt);  // (the table was written a step ago)
+      // the activation tile of three steps on, into the ring slot everyone finished reading before the barrier above
+      if (step + kPAhead < n_steps) {
+        const int slot = (step + kPAhead) & (kPARing - 1);
+        if (ks + kPAhead < nks) move_a(slot, ks + kPAhead, arow_off);
+        else move_a(slot, ks + kPAhead - nks, arow_nxt);
+      }
+      if (nb > 0) {
+        const _Float16* pa = sA + (step & (kPARing - 1)) * kPM * kPK + (32 * wm + (lane & 31)) * kPK;
+        const _Float16* pb = sB + (step & 1) * kPR * kPK + (wq * 64 + (lane & 31)) * kPK;
+        const int aswz = pc_swizzle(lane), khalf = lane >> 5;    // (block rows start at multiples of 32: the row's low bits are the lane's)
+        const int wswz = aswz;
+        half8 fa[2][2], fb[2][2];
+        auto frags = [&](int kk, int set) __attribute__((always_inline)) {
+          const int apos = ((kk * 2 + khalf) ^ aswz) * 8, bpos = ((kk * 2 + khalf) ^ wswz) * 8;
+#pragma unroll
+          for (int mi = 0; mi < 2; ++mi)
+            if (mi < nb) fa[set][mi] = *reinterpret_cast<const half8*>(pa + mi * 64 * kPK + apos);
+#pragma unroll
+          for (int ni = 0; ni < 2; ++ni) fb[set][ni] = *reinterpret_cast<const half8*>(pb + ni * 32 * kPK + bpos);
+        };
+        frags(0, 0);
+#pragma unroll
+        for (int kk = 0; kk < kPK / 16; ++kk) {
+          const int c = kk & 1;
+          if (kk + 1 < kPK / 16) frags(kk + 1, c ^ 1);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int mi = 0; mi < 2; ++mi) {
+            if (mi < nb) {
+#pragma unroll
+              for (int ni = 0; ni < 2; ++ni)
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[c][mi], fb[c][ni], acc[mi][ni], 0, 0, 0);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+
+    // epilogue: acc[mi][ni][v] is tile row 32 (2 mi + wm) + (v / 4) * 8 + (lane / 32) * 4 + v % 4, column lane % 32 of
+    // the wavefront's column block ni
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+      if (mi >= nb) break;
+      int orows[16];
+      [[maybe_unused]] float scs[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int r = 32 * (2 * mi + wm) + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+        orows[v] = sOrow[tb * kTable + r];
+        if (NM == 1) scs[v] = sScale[tb * kTable + r];
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int orow = orows[v];
+        if (orow < 0) continue;
+        if (NM == 2) {
+          // column blocks 0 and 1: gate and the matching up columns
+          const int col = cur.nt * (kPR / 2) + wq * 32 + (lane & 31);
+          const float g = acc[mi][0][v] * kWScaleInv, u = acc[mi][1][v] * kWScaleInv;
+          static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_f(g) * u);
+        } else {
+#pragma unroll
+          for (int ni = 0; ni < 2; ++ni) {
+            const int col = cur.nt * kPR + wq * 64 + ni * 32 + (lane & 31);
+            static_cast<float*>(a.out)[(size_t)orow * a.n_rows + col] = scs[v] * (acc[mi][ni][v] * kWScaleInv);
+          }
+        }
+      }
+    }
+    cur = nxt;
+#pragma unroll
+    for (int i = 0; i < kPAInstr; ++i) arow_off[i] = arow_nxt[i];
+  }
+}
+
 // fp32 -> fp16 activations for live rows; rows past `valid` are left alone.
 __global__ void __launch_bounds__(256) k_to_f16_rows(const float* __restrict__ x, const int* __restrict__ valid_tokens,
                                                       int width, _Float16* __restrict__ out) {
@@ -719,11 +1117,15 @@ bool mfma_supported(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int ga
 // 702 against 695 us at 2048 tokens).
 // `tokens`: pass_tokens() below.
 static int routed_tile_rows(const xabe_moe_geometry& g, size_t tokens) {
-#ifdef XABE_TILE_ENV
-  if (const char* e = getenv("XABE_BM")) return atoi(e);
-#endif
   return tokens * g.experts_per_token <= 48 * g.num_experts ? 64 : kBM;
 }
+// The specialised form (k_mfma_pc) serves both routed launches for contractions of whole superblocks and at least
+// eight steps, when asked for: `mfma_form` 2 (0 and 1: k_mfma_expert everywhere; it is the faster at every width
+// measured, see k_mfma_pc).
+static bool pc_shape_ok(const xabe_moe_geometry& g) {
+  return g.hidden % 256 == 0 && g.intermediate % 256 == 0 && g.hidden >= 512 && g.intermediate >= 512;
+}
+static bool pc_form(const xabe_moe_kernels* k, size_t) { return k->mfma_form == 2 && pc_shape_ok(k->g); }
 // The tokens a pass is known to hold when its launches are chosen: the live count last published to the device
 // scalar (a 512-token chunk run in buffers sized for 8192 should get the tiles of a 512-token pass), the buffers'
 // size before any was.  Every tile height serves any live count and gives the same bits, so a graph captured at one
@@ -736,10 +1138,9 @@ static size_t pass_tokens(const xabe_moe_kernels* k, const xabe_moe_buffers* b) 
 // -> 1263 us (the launch itself 503 -> ~415), 6144 tokens 1081 -> 1043; at 4096 tokens (128 per expert) the tall tile
 // loses (778 against 767).  The down launch keeps the short tiles at every width: its contraction is four steps, its
 // items are mostly epilogue, and with tall tiles the block measured 1279 us against 1263.
-static int routed_up_tile_rows(const xabe_moe_geometry& g, size_t tokens) {
-#ifdef XABE_TILE_ENV
-  if (const char* e = getenv("XABE_BM_UP")) return atoi(e);
-#endif
+static int routed_up_tile_rows(const xabe_moe_kernels* k, size_t tokens) {
+  const xabe_moe_geometry& g = k->g;
+  if (pc_form(k, tokens)) return kPM;
   if (tokens * g.experts_per_token >= 192 * g.num_experts) return 384;
   return routed_tile_rows(g, tokens);
 }
@@ -753,7 +1154,8 @@ bool mfma_tile_plan(const xabe_moe_kernels* k, const xabe_moe_buffers* b, int* b
   if (!b->tile_list || b->n_tile_list < 16 || !k->tensor_cores || k->exact_regime) return false;
   const size_t tokens = pass_tokens(k, b);
   *bm = routed_tile_rows(k->g, tokens);
-  *bm_up = routed_up_tile_rows(k->g, tokens);
+  if (pc_form(k, tokens)) *bm = kPM;  // (both specialised launches: 128-row tiles, one list)
+  *bm_up = routed_up_tile_rows(k, tokens);
   *capacity = (int)((b->n_tile_list / 2 - 4) / 4);
   return true;
 }
@@ -772,9 +1174,28 @@ static int configure_one() {
     XABE_HIP_TRY(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)mfma_lds_bytes<TBM>()));
   return XABE_OK;
 }
+template <int NM>
+static int configure_pc() {
+  const void* fns[2] = {reinterpret_cast<const void*>(k_mfma_pc<kQ6K, NM>), reinterpret_cast<const void*>(k_mfma_pc<kQ8_0, NM>)};
+  for (const void* f : fns)
+    XABE_HIP_TRY(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)mfma_pc_lds_bytes()));
+  return XABE_OK;
+}
+template <int NM>
+static int launch_pc(const xabe_moe_kernels* k, int quant, const MfmaArgs& a, size_t max_items, hipStream_t s) {
+  const unsigned grid = (unsigned)std::max<size_t>(1, std::min<size_t>(max_items, (size_t)k->num_cus));  // one workgroup per CU
+  constexpr size_t smem = mfma_pc_lds_bytes();
+  if (quant == XABE_QUANT_Q6K) hipLaunchKernelGGL((k_mfma_pc<kQ6K, NM>), dim3(grid), dim3(1024), smem, s, a);
+  else hipLaunchKernelGGL((k_mfma_pc<kQ8_0, NM>), dim3(grid), dim3(1024), smem, s, a);
+  XABE_HIP_TRY(hipGetLastError());
+  return XABE_OK;
+}
+
 int mfma_configure() {
   static bool done = false;  // (one device per process)
   if (done) return XABE_OK;
+  XABE_TRY((configure_pc<2>()));
+  XABE_TRY((configure_pc<1>()));
   XABE_TRY((configure_one<1, false, 64>()));
   XABE_TRY((configure_one<1, false, 128>()));
   XABE_TRY((configure_one<1, true, 64>()));
@@ -851,7 +1272,9 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   a.out = b->inter_h;
   a.K = (int)g.hidden;
   a.n_rows = (int)g.intermediate;
-  if (bm_up == 64) XABE_TRY((launch_mfma<2, true, 64>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
+  const bool pc = pc_form(k, pass_tokens(k, b));
+  if (pc && bm_up == kPM) XABE_TRY((launch_pc<2>(k, gate.quant, a, max_mtiles * (g.intermediate / (kPR / 2)), s)));
+  else if (bm_up == 64) XABE_TRY((launch_mfma<2, true, 64>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
   else if (bm_up == 384) XABE_TRY((launch_mfma<2, true, 384>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
   else XABE_TRY((launch_mfma<2, true, 128>(k, gate.quant, a, max_mtiles * (g.intermediate / 64), s)));
   // down -> partial[flat][H], scaled by the routing weight
@@ -863,7 +1286,8 @@ int mfma_grouped_forward_partial(const xabe_moe_kernels* k, hipStream_t s, xabe_
   a.out = b->partial;
   a.K = (int)g.intermediate;
   a.n_rows = (int)g.hidden;
-  if (bm == 64) XABE_TRY((launch_mfma<1, true, 64>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
+  if (pc && bm == kPM) XABE_TRY((launch_pc<1>(k, down.quant, a, max_mtiles * (g.hidden / kPR), s)));
+  else if (bm == 64) XABE_TRY((launch_mfma<1, true, 64>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
   else XABE_TRY((launch_mfma<1, true, 128>(k, down.quant, a, max_mtiles * (g.hidden / 128), s)));
   return XABE_OK;
 }

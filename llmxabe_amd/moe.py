@@ -223,6 +223,10 @@ class MoeKernels:
     def disable_tensor_cores(self): check(_ffi.lib().xabe_moe_kernels_disable_tensor_cores(self._h))
     def tensor_cores_enabled(self) -> bool: return bool(_ffi.lib().xabe_moe_kernels_tensor_cores_enabled(self._h))
     def force_community(self, on: bool): check(_ffi.lib().xabe_moe_kernels_force_community(self._h, int(on)))
+    def set_mfma_form(self, form: int):
+        """0: by width; 1: k_mfma_expert; 2: k_mfma_pc wherever the shape allows (a comparison switch; see the header)."""
+        check(_ffi.lib().xabe_moe_kernels_set_mfma_form(self._h, form))
+
     def set_exact_decode_regime(self, on: bool): check(_ffi.lib().xabe_moe_kernels_set_exact_decode_regime(self._h, int(on)))
 
     def set_valid_tokens(self, buffers: MoeBuffers, tokens: int):

@@ -466,3 +466,38 @@ def test_router_logits_matrix_core_path(oracle, X, router_q8):
     rows = np.r_[0:40, 1000:1040, live - 40:live]
     want = normed.cpu().numpy()[rows].astype(np.float64) @ w.astype(np.float64).T
     assert rel_to_peak(got[rows], want) <= 2e-5
+
+
+@pytest.mark.parametrize("tokens,quant", [(8192, "q6k"), (5000, "q6k"), (3072, "q6k"), (1024, "q6k"), (8192, "q8_0"), (640, "q8_0")])
+def test_specialised_wavefronts_give_the_bits_of_the_plain_kernel(oracle, X, tokens, quant):
+    """k_mfma_pc (half of a workgroup's wavefronts multiply, half dequantise; 64-element steps; 128-row x 256-weight-row
+    tiles; selected with set_mfma_form(2)) against k_mfma_expert on the same pass: every output element sees the same
+    fp16 operands in the same order of matrix instructions, so `partial` and the reduced rows are the same bits.
+    Several widths, a ragged live count, both formats."""
+    import torch
+
+    q = X.ExpertQuant.Q6K if quant == "q6k" else X.ExpertQuant.Q8_0
+    T = max(tokens, 64)
+    g = X.MoeGeometry.qwen3_6(X.moe_block_size(T), T)
+    layer = make_layer(oracle, g, seed=736, expert_quant=q)
+    d = layer.dev
+    rng = np.random.default_rng(tokens)
+    logits = torch.from_numpy(rng.uniform(-3, 3, (T, 256)).astype(np.float32)).cuda()
+    x = activations(39, T, 2048)
+    live = tokens - 3
+    outs = []
+    for form in (1, 2):
+        k = X.MoeKernels(g)
+        k.set_mfma_form(form)
+        b = k.buffers()
+        k.set_valid_tokens(b, live)
+        k.route_and_dispatch(b, logits)
+        out = torch.zeros(T, 2048, device="cuda")
+        k.grouped_forward(b, d.gate_exps, d.up_exps, d.down_exps, x, out)
+        torch.cuda.synchronize()
+        outs.append((out, b.partial().clone()))
+        del k, b
+    assert float(outs[0][0][:live].abs().max()) > 0
+    assert torch.equal(outs[0][0].view(torch.int32), outs[1][0].view(torch.int32))
+    n = live * 8 * 2048
+    assert torch.equal(outs[0][1][:n].view(torch.int32), outs[1][1][:n].view(torch.int32))
