@@ -161,6 +161,20 @@ int long_rows_configure() {
                         reinterpret_cast<const void*>(k_shared_long_rows<kQ8_0, 2, 2, 4, false, true>)};
   for (const void* f : fns)
     XABE_HIP_TRY(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongRowsLdsMax));
+  const void* staged[6] = {reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 2, 2, false>),
+                           reinterpret_cast<const void*>(k_long_rows_staged<kQ8_0, 2, 2, false>),
+                           reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 1, 4, false>),
+                           reinterpret_cast<const void*>(k_long_rows_staged<kQ8_0, 1, 4, false>),
+                           reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 1, 4, true>),
+                           reinterpret_cast<const void*>(k_long_rows_staged<kQ8_0, 1, 4, true>)};
+  const void* staged10[4] = {reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 1, 2, false, 10>),
+                             reinterpret_cast<const void*>(k_long_rows_staged<kQ8_0, 1, 2, false, 10>),
+                             reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 1, 2, true, 10>),
+                             reinterpret_cast<const void*>(k_long_rows_staged<kQ8_0, 1, 2, true, 10>)};
+  for (const void* f : staged10)
+    XABE_HIP_TRY(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStagedLdsBytes));
+  for (const void* f : staged)
+    XABE_HIP_TRY(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStagedLdsBytes));
   done = true;
   return XABE_OK;
 }
@@ -187,6 +201,30 @@ bool launch_long_rows(const xabe_moe_kernels* k, int quant, int nm, const LongRo
   const size_t row_bytes = (size_t)a.K / xabe_expert_quant_block_elements(quant) * xabe_expert_quant_block_bytes(quant);
   auto on16 = [&](const uint8_t* w) { return !w || (reinterpret_cast<uintptr_t>(w) % 16 == 0 && ((size_t)a.n_rows * row_bytes) % 16 == 0); };
   if (!(on16(a.w0) && on16(a.w1))) return false;
+  // Five tokens or more: eight tokens per pass, the step's activations staged in LDS for the whole workgroup
+  // (k_long_rows_staged); one workgroup of eight wavefronts per CU, persistent over groups of 8 r rows.
+  if (k->g.max_tokens >= 5 && a.n_rows % (8 * r) == 0 && a.K % 256 == 0 &&
+      (size_t)k->g.max_tokens * (size_t)a.K * sizeof(float) < ((size_t)1 << 32) && reinterpret_cast<uintptr_t>(a.x) % 16 == 0) {
+    const unsigned pass8 = (unsigned)((k->g.max_tokens + kStagedTok - 1) / kStagedTok);
+    const unsigned groups8 = (unsigned)(a.n_rows / (8 * r));
+    dim3 grid8(std::min<unsigned>(groups8, (unsigned)k->num_cus), pass8), block8(512);
+    // a single matrix whose groups of 32 rows leave CUs idle while groups of 20 fill them (the dense sibling's down
+    // projection: 5120 rows, 160 against 256 groups): ten wavefronts of two rows
+    const bool ten = nm == 1 && a.n_rows % 20 == 0 && groups8 < (unsigned)k->num_cus && (unsigned)(a.n_rows / 20) >= groups8 * 3 / 2;
+    const dim3 grid10(std::min<unsigned>((unsigned)(a.n_rows / 20), (unsigned)k->num_cus), pass8), block10(640);
+#define XABE_STAGED(Q)                                                                                                          \
+  do {                                                                                                                          \
+    if (nm == 2) hipLaunchKernelGGL((k_long_rows_staged<Q, 2, 2, false>), grid8, block8, kStagedLdsBytes, s, la);               \
+    else if (ten && resid) hipLaunchKernelGGL((k_long_rows_staged<Q, 1, 2, true, 10>), grid10, block10, kStagedLdsBytes, s, la); \
+    else if (ten) hipLaunchKernelGGL((k_long_rows_staged<Q, 1, 2, false, 10>), grid10, block10, kStagedLdsBytes, s, la);        \
+    else if (resid) hipLaunchKernelGGL((k_long_rows_staged<Q, 1, 4, true>), grid8, block8, kStagedLdsBytes, s, la);             \
+    else hipLaunchKernelGGL((k_long_rows_staged<Q, 1, 4, false>), grid8, block8, kStagedLdsBytes, s, la);                       \
+  } while (0)
+    if (quant == XABE_QUANT_Q6K) XABE_STAGED(kQ6K);
+    else XABE_STAGED(kQ8_0);
+#undef XABE_STAGED
+    return true;
+  }
   // Three tokens or more, gate/up: four tokens per pass with the activation rows in LDS (the kernel's XLDS form),
   // where four rows and eight wavefronts' staging slots fit; eight wavefronts per workgroup, one workgroup per
   // CU and pass, persistent over the row groups.  (Down's rows are too long for four of them to fit.)

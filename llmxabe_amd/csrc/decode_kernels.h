@@ -742,6 +742,226 @@ __global__ void __launch_bounds__(XLDS ? 512 : 256) k_shared_long_rows(LongRowAr
   }
 }
 
+// The long-row kernel for five to eight tokens in ONE pass over the weights (more tokens: further passes of eight).
+// With a lane's 32 activations per token held in registers a pass serves two tokens, or four with the rows in LDS
+// (k_shared_long_rows); the dense sibling's down projection then reads its 73 MB four times at eight tokens.  Here
+// the step's activations of all eight tokens (2048 elements each) are staged in LDS, double-buffered, by
+// global -> LDS DMA in the order the lanes consume them ([place j][word w][token][lane] as 16-byte slots, conflict
+// free), and a wavefront runs R rows (or gate/up pairs) against them with the work ordered place-major: for one
+// place j the eight tokens' four activations of word w sit in 32 registers while every row's codes of that place
+// are converted once and multiplied for all eight tokens.  Per (row, token) this is q6_accum's / q8_accum's
+// sequence of operations exactly (acc_j: word 0's four products, then word 1's; tot += ds_j * (acc_j + xs_j) for
+// j = 0..3; Q8_0: one accumulator over the eight words, tot += d * acc), the lane partial carried step after step
+// and reduced once: the bits of k_shared_long_rows and of single-token decode.
+// A workgroup is eight (or ten) wavefronts (wavefront w < 8 issues the DMA of place-word w), one per CU (144 KB of
+// LDS), persistent over row groups of WAVES x R rows; the (group, step) sequence is one pipeline: while a step is multiplied
+// the next step's activations and raw weight bytes are in flight.  Two barriers per step: the DMA has landed
+// everywhere; the run sums (-32 * sum of each eight, Q6_K's code offset) have been formed from it, and lanes past
+// the end of a row's last step zeroed.
+constexpr int kStagedTok = 8;
+constexpr size_t kStagedLdsBytes = 2 * (8 * kStagedTok * 64 * 16 + 4 * kStagedTok * 64 * 4);
+
+// WAVES: wavefronts per workgroup, eight or ten (ten x two rows = twenty rows per group gives the down projection's
+// 5120 rows one group per CU, where eight x four leave 96 of 256 CUs without work).
+template <int QUANT, int NM, int R, bool RESID, int WAVES = 8>
+__global__ void __launch_bounds__(64 * WAVES, WAVES > 8 ? 3 : 2) k_long_rows_staged(LongRowArgs la) {
+  using F = Fmt<QUANT>;
+  using Raw = typename F::Raw;
+  constexpr int TOK = kStagedTok, RW = R * NM;
+  extern __shared__ __attribute__((aligned(16))) uint8_t s_staged[];
+  float4* const s_xq = reinterpret_cast<float4*>(s_staged);               // [2][8][TOK][64]
+  float* const s_xs = reinterpret_cast<float*>(s_xq + 2 * 8 * TOK * 64);  // [2][4][TOK][64]
+  const ExpertArgs& a = la.m;
+  const int valid = *a.valid_tokens;
+  const int t0 = blockIdx.y * TOK;
+  if (t0 >= valid) return;
+  const int nt = min(TOK, valid - t0);
+  const LaneGeom g = lane_geom<QUANT>();
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const size_t row_bytes = (size_t)(a.K / F::kBlockElems) * F::kBlockBytes;
+  const int steps = (a.K + kStepElems - 1) / kStepElems;
+  const int n_groups = a.n_rows / (WAVES * R);
+  if ((int)blockIdx.x >= n_groups) return;
+  const int n_mine = (n_groups - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int total = n_mine * steps;
+
+  // DMA of step s into buffer b: this wavefront's place-word (j = wave >> 1, w = wave & 1) of all tokens
+  const uint32_t lds_x = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)s_xq;
+  auto stage = [&](int s, int b) __attribute__((always_inline)) {
+    if (WAVES > 8 && wave >= 8) return;
+    const int koff = min(lane_koff<QUANT, 1>(g, s), a.K - F::kBlockElems);
+    const int j = wave >> 1, w = wave & 1;
+    const int e = QUANT == kQ6K ? koff + g.half * 128 + j * 32 + g.l8 * 8 + w * 4 : koff + j * 8 + w * 4;
+#pragma unroll
+    for (int t = 0; t < TOK; ++t) {
+      const uint32_t voff = (uint32_t)(((size_t)(t0 + min(t, nt - 1)) * a.K + e) * sizeof(float));
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_x + (uint32_t)(((b * 8 + wave) * TOK + t) * 64 * 16));
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(a.x), "s"(dst) : "memory", "m0");
+#pragma clang diagnostic pop
+    }
+  };
+  // run sums of buffer b (step s), and zeros for the lanes past the end of the row: four runs per thread
+  auto finish_stage = [&](int s, int b) __attribute__((always_inline)) {
+    constexpr int kRuns = 4 * kStagedTok * 64, kThreads = 64 * WAVES;
+#pragma unroll
+    for (int i = 0; i < (kRuns + kThreads - 1) / kThreads; ++i) {
+      const int r = (int)threadIdx.x + kThreads * i, ln = r & 63, t = (r >> 6) & 7, j = r >> 9;
+      if (kRuns % kThreads != 0 && r >= kRuns) break;
+      const int koff = QUANT == kQ6K ? ((ln >> 3) + s * 8) * 256 : (ln + s * 64) * 32;
+      const bool act = koff < a.K;
+      float4* p0 = s_xq + ((b * 8 + 2 * j) * TOK + t) * 64 + ln;
+      float4* p1 = p0 + TOK * 64;
+      float4 v0 = *p0, v1 = *p1;
+      if (!act) {
+        v0 = v1 = make_float4(0.f, 0.f, 0.f, 0.f);
+        *p0 = v0;
+        *p1 = v1;
+      }
+      if constexpr (QUANT == kQ6K) {
+        float sum = 0.0f;  // (the order of lane_x_offsets)
+        sum += v0.x; sum += v0.y; sum += v0.z; sum += v0.w;
+        sum += v1.x; sum += v1.y; sum += v1.z; sum += v1.w;
+        s_xs[((b * 4 + j) * TOK + t) * 64 + ln] = -32.0f * sum;
+      }
+    }
+  };
+  auto load_rows = [&](int grp, int s, Raw (&raw)[RW]) __attribute__((always_inline)) {
+    const bool act = lane_koff<QUANT, 1>(g, s) < a.K;
+    const int row0 = (grp * WAVES + wave) * R;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const size_t off = (size_t)(row0 + r) * row_bytes + (size_t)s * F::kChunkBytes;
+      load_raw<QUANT, true>(a.w0 + off, act, g, raw[r * NM]);
+      if constexpr (NM == 2) load_raw<QUANT, true>(a.w1 + off, act, g, raw[r * NM + NM - 1]);
+    }
+  };
+
+  Raw raw_next[RW];
+  stage(0, 0);
+  load_rows((int)blockIdx.x, 0, raw_next);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  finish_stage(0, 0);
+  __syncthreads();
+
+  float tot[RW][TOK];
+#pragma unroll
+  for (int rw = 0; rw < RW; ++rw)
+#pragma unroll
+    for (int t = 0; t < TOK; ++t) tot[rw][t] = 0.0f;
+  int grp = (int)blockIdx.x, s = 0;
+#pragma unroll 1
+  for (int i = 0; i < total; ++i) {
+    const int b = i & 1;
+    Raw raw[RW];
+#pragma unroll
+    for (int rw = 0; rw < RW; ++rw) raw[rw] = raw_next[rw];
+    const int s_n = s + 1 < steps ? s + 1 : 0, grp_n = s + 1 < steps ? grp : grp + (int)gridDim.x;
+    if (i + 1 < total) {
+      stage(s_n, b ^ 1);
+      load_rows(grp_n, s_n, raw_next);
+      issue_fence();
+    }
+    // ---- this step, place-major
+    const float4* xq = s_xq + (size_t)b * 8 * TOK * 64 + g.lane;
+    const float* xsb = s_xs + (size_t)b * 4 * TOK * 64 + g.lane;
+    float accj[RW][TOK];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (QUANT == kQ6K || j == 0) {
+#pragma unroll
+        for (int rw = 0; rw < RW; ++rw)
+#pragma unroll
+          for (int t = 0; t < TOK; ++t) accj[rw][t] = 0.0f;
+      }
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        float4 xv[TOK];
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) xv[t] = xq[((2 * j + w) * TOK + t) * 64];
+#pragma unroll
+        for (int rw = 0; rw < RW; ++rw) {
+          float f0, f1, f2, f3;
+          if constexpr (QUANT == kQ6K) {
+            const Q6Raw& r = raw[rw];
+            const uint32_t qa = w ? r.qa1 : r.qa0, qb = w ? r.qb1 : r.qb0, qh = w ? r.qh1 : r.qh0;
+            const uint32_t c = j == 0   ? (qa & 0x0F0F0F0Fu) | ((qh << 4) & 0x30303030u)
+                               : j == 1 ? (qb & 0x0F0F0F0Fu) | ((qh << 2) & 0x30303030u)
+                               : j == 2 ? ((qa >> 4) & 0x0F0F0F0Fu) | (qh & 0x30303030u)
+                                        : ((qb >> 4) & 0x0F0F0F0Fu) | ((qh >> 2) & 0x30303030u);
+            f0 = ub0(c), f1 = ub1(c), f2 = ub2(c), f3 = ub3(c);
+          } else {
+            const uint32_t c = raw[rw].q[2 * j + w];
+            f0 = sb0(c), f1 = sb1(c), f2 = sb2(c), f3 = sb3(c);
+          }
+#pragma unroll
+          for (int t = 0; t < TOK; ++t) {
+            float v = accj[rw][t];
+            v = __builtin_fmaf(f0, xv[t].x, v);
+            v = __builtin_fmaf(f1, xv[t].y, v);
+            v = __builtin_fmaf(f2, xv[t].z, v);
+            v = __builtin_fmaf(f3, xv[t].w, v);
+            accj[rw][t] = v;
+          }
+        }
+      }
+      if constexpr (QUANT == kQ6K) {
+        float xsj[TOK];
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) xsj[t] = xsb[(j * TOK + t) * 64];
+        const int is8 = (g.l8 >> 1) * 8;
+#pragma unroll
+        for (int rw = 0; rw < RW; ++rw) {
+          const uint32_t sw = (j < 2 ? raw[rw].sc0 : raw[rw].sc1) >> is8;
+          const float ds = f16_bits_to_f32(raw[rw].dh) * (float)(int8_t)((j & 1 ? sw >> 16 : sw) & 0xff);
+#pragma unroll
+          for (int t = 0; t < TOK; ++t) tot[rw][t] = __builtin_fmaf(ds, accj[rw][t] + xsj[t], tot[rw][t]);
+        }
+      }
+    }
+    if constexpr (QUANT != kQ6K) {
+#pragma unroll
+      for (int rw = 0; rw < RW; ++rw) {
+        const float d = f16_bits_to_f32(raw[rw].dh);
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) tot[rw][t] = __builtin_fmaf(d, accj[rw][t], tot[rw][t]);
+      }
+    }
+    if (s == steps - 1) {
+      // the group's rows are complete: reduce over the lanes once, store, start over
+      const int row0 = (grp * WAVES + wave) * R;
+#pragma unroll
+      for (int t = 0; t < TOK; ++t) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          float red[NM];
+#pragma unroll
+          for (int m = 0; m < NM; ++m) red[m] = group_sum<64>(tot[r * NM + m][t]);
+          if (g.lane == 0 && t < nt) {
+            const size_t o = (size_t)(t0 + t) * a.n_rows + row0 + r;
+            const float v = NM == 2 ? silu_f(red[0]) * red[NM - 1] : 1.0f * red[0];
+            a.out[o] = v;
+            if constexpr (RESID) la.l_out[o] = v + la.residual[o];
+          }
+        }
+      }
+#pragma unroll
+      for (int rw = 0; rw < RW; ++rw)
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) tot[rw][t] = 0.0f;
+    }
+    // the next step's activations have landed (requested a whole step ago) and everyone is done with this buffer
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (i + 1 < total) finish_stage(s_n, b ^ 1);
+    __syncthreads();
+    s = s_n;
+    grp = grp_n;
+  }
+}
+
 template <int QUANT, int KS, int RPS, int NM>
 __global__ void __launch_bounds__(256) k_expert_shared(ExpertArgs a) {
   shared_body<QUANT, KS, RPS, NM>(a, blockIdx.y, blockIdx.x);
