@@ -26,13 +26,6 @@
 
 #include "decode_kernels.h"
 #include "host_common.h"
-#ifdef XABE_TRACE_ITEMS
-namespace xabe { static __device__ long long g_route_trace[4096 * 8]; }
-#define XABE_ROUTE_TRACE(slot)                                                                              \
-  do {                                                                                                      \
-    if ((threadIdx.x & 63) == 0 && blockIdx.x < 4096) xabe::g_route_trace[blockIdx.x * 8 + (slot)] = wall_clock64(); \
-  } while (0)
-#endif
 #include "route_device.h"
 
 namespace xabe {
@@ -71,16 +64,6 @@ constexpr int kMaxInter = 512;    // intermediate width staged in LDS by k_decod
 constexpr int kDownSteps = 2;
 static int logits_depth(int max_tokens) { return max_tokens <= 1 ? 1 : max_tokens <= 6 ? 2 : 4; }
 
-#ifdef XABE_TRACE_ITEMS
-// measurement builds only: per-workgroup timestamps (100 MHz device clock), [kernel][workgroup][slot]
-static __device__ long long g_item_trace[3 * 4096 * 4];
-#define XABE_TRACE(kernel, slot)                                                                          \
-  do {                                                                                                    \
-    if (threadIdx.x == 0 && blockIdx.x < 4096) g_item_trace[((kernel) * 4096 + blockIdx.x) * 4 + (slot)] = wall_clock64(); \
-  } while (0)
-#else
-#define XABE_TRACE(kernel, slot) do { } while (0)
-#endif
 
 struct DecodeArgs {
   const float* residual;
@@ -243,7 +226,6 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
   const int chunks = (a.max_tokens + 1) / 2;
   const int n_r = chunks * a.tiles_r;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  XABE_TRACE(0, 0);
   if ((int)blockIdx.x >= a.max_tokens) {
     int item = blockIdx.x - a.max_tokens;
     const bool router = item < n_r;
@@ -271,7 +253,6 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
         tile_normed<SQ, RPS, 1, 2, kLogitsDepth, PRE>(a.sgate, a.sup, a.H, a.I, row0, xr, a.post_norm, a.eps, o, nullptr, a.valid_tokens, t0, s_xn);
       }
     }
-    XABE_TRACE(0, 3);
     return;
   }
   // the normalised row (callers read it back) and g = sigmoid(shared_gate_inp . normed): the order of
@@ -310,7 +291,6 @@ __global__ void __launch_bounds__(256) k_decode_logits(DecodeArgs a) {
   __syncthreads();
   const float total = ((s_red[0] + s_red[1]) + s_red[2]) + s_red[3];
   if (threadIdx.x == 0) a.gate_out[t] = 1.0f / (1.0f + expf(-total));
-  XABE_TRACE(0, 2);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -356,7 +336,6 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const LaneGeom g = lane_geom<RQ>();
   const int koff = lane_koff<RQ, RPS>(g, 0);
-  XABE_TRACE(1, 0);
   // one wavefront routes the token (a different one in neighbouring workgroups, which share a CU); its
   // logits and every wavefront's copy of the normalised row are requested together
   const bool routes = !ROUTED && wave == (int)((blockIdx.x >> 8) & 3);
@@ -380,7 +359,6 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   int cand_i = 0;
   int key[kRouteMaxPerLane];
   if (routes) {
-    XABE_ROUTE_TRACE(0);
     if (few) {
       route_keys<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, *reinterpret_cast<int(*)[4]>(key));
       route_rounds<4>(*reinterpret_cast<int(*)[4]>(key), 0, k + 1, cand_i);
@@ -392,7 +370,6 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
   }
   lane_x_offsets<RQ>(x[0], xs[0]);
   if constexpr (!ROUTED) __syncthreads();
-  XABE_TRACE(1, 1);
   const size_t row_bytes = (size_t)(a.H / F::kBlockElems) * F::kBlockBytes;
   const int wave_row0 = (tile * kWavesPerWg + wave) * DEPTH * RPS;
   float* out = a.inter + (size_t)p * a.I;
@@ -424,7 +401,6 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
         else route_rounds<kRouteMaxPerLane>(key, k + 1, n_cand, cand_i);
         if (few) route_finish<4>(*reinterpret_cast<float(*)[4]>(lg), a.E, a.top_k, n_cand, cand_i, s_route, sel_i, sel_w, exact);
         else route_finish<kRouteMaxPerLane>(lg, a.E, a.top_k, n_cand, cand_i, s_route, sel_i, sel_w, exact);
-        XABE_ROUTE_TRACE(5);
         if (g.lane == k) s_final = sel_i;
         if (k == 0 && tile == 0 && g.lane < a.top_k) {
           a.topk_ids[(size_t)t * a.top_k + g.lane] = sel_i;
@@ -436,7 +412,6 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
     request(0, DEPTH);  // (the other wavefronts come straight here)
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      if (d == 1) XABE_TRACE(1, 2);
       float tg[1] = {0.0f}, tu[1] = {0.0f};
       accum<RQ, 1>(r[d][0], g, x, xs, tg);
       accum<RQ, 1>(r[d][1], g, x, xs, tu);
@@ -454,7 +429,6 @@ __global__ void __launch_bounds__(256) k_decode_up(DecodeArgs a) {
     const int e_final = s_final;
     if (e_final != e) stream_rows(e_final, std::false_type{});  // (same rows of `inter`, written again)
   }
-  XABE_TRACE(1, 3);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -491,7 +465,6 @@ __global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
   const int rs = wave >> 1, second = wave & 1;
   const int lane = __lane_id();
   const int row0 = (tile * RS + rs) * RPS;  // hidden is a multiple of RS * RPS
-  XABE_TRACE(2, 0);
   // this wavefront's selections: [k0, k1)
   const int split = (a.top_k + 1) / 2;
   const int k0 = second ? split : 0, k1 = second ? a.top_k : split;
@@ -556,7 +529,6 @@ __global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
     }
   }
   __syncthreads();
-  XABE_TRACE(2, 1);
   // x[32] of one staged row for this lane, and (Q6_K) the four run sums that go with them
   auto lane_x = [&](auto quant_c, int slot, const LaneGeom& g, float (&x)[1][32], float (&xs)[1][4]) __attribute__((always_inline)) {
     constexpr int Q = decltype(quant_c)::value;
@@ -577,7 +549,6 @@ __global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
       part[j] = sel_w[j] * group_sum<G>(tot[0]);
     }
   }
-  XABE_TRACE(2, 2);
   const bool writes = (lane % G) == 0;
   if (second) {
     if (writes) {
@@ -613,7 +584,6 @@ __global__ void __launch_bounds__(128 * RS) k_decode_down(DecodeArgs a) {
     if (a.next_normed) __hip_atomic_store(a.l_out + i, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     else a.l_out[i] = lo;
   }
-  XABE_TRACE(2, 3);
   if (!a.next_normed) return;
   // The seam (docs/BENCHMARKS.md:1376 of the reference: the next layer's RMSNorm in the combine's tail).  A token's
   // row is finished by tiles_d workgroups, and the wavefront that finishes it last applies the norm.  Arrivals are
@@ -824,12 +794,3 @@ int launch_decode_block(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffe
 }
 
 }  // namespace xabe
-
-#ifdef XABE_TRACE_ITEMS
-extern "C" int xabe_debug_read_route_trace(long long* out, size_t n) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(xabe::g_route_trace), n * sizeof(long long));
-}
-extern "C" int xabe_debug_read_item_trace(long long* out, size_t n) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(xabe::g_item_trace), n * sizeof(long long));
-}
-#endif

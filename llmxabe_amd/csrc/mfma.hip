@@ -200,17 +200,6 @@ __device__ __forceinline__ void load_step_w(int ks, const uint8_t* const (&wrow)
   for (int i = 0; i < UNITS; ++i) load_unit_w<QUANT, UNITS>(ks, i, wrow, du, wreg);
 }
 
-#ifdef XABE_MFMA_TRACE
-// measurement builds only: [workgroup < 512][step slot < 32][4 stamps] of the routed gate/up launch (100 MHz clock)
-static __device__ long long g_mfma_trace[512 * 32 * 4];
-#define XABE_MT(slot)                                                                                             \
-  do {                                                                                                            \
-    if (NM == 2 && ROUTED && tid == 0 && blockIdx.x < 512 && trace_step < 32)                                     \
-      g_mfma_trace[(blockIdx.x * 32 + trace_step) * 4 + (slot)] = wall_clock64();                                 \
-  } while (0)
-#else
-#define XABE_MT(slot) do { } while (0)
-#endif
 
 // TBM: token rows per tile, 384, 128 or 64.  The narrow form serves geometries whose experts see at most ~64 tokens
 // each (up to ~2000 tokens per pass): half the matrix instructions, activation bytes and output stores per
@@ -262,7 +251,6 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_m
   // dequant mapping: unit u of LDS weight rows rb0 and rb0 + 64
   const int du = tid & 3, rb0 = tid >> 2;
 
-  [[maybe_unused]] int trace_step = 0;
   // Which items this workgroup takes.  Workgroup ids are dealt round-robin to the eight XCDs, each with its
   // own L2: when there is work for every workgroup, XCD x takes a contiguous eighth of the token tiles and its
   // workgroups walk that range together (token tile major), so an activation tile is fetched into one L2
@@ -444,7 +432,6 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_m
       order_fence();
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       order_fence();
-      XABE_MT(0);
       if constexpr (ROUTED && NM == 1) {
         // the next item's output scales, two steps before they are stored.  (First thing in the step: the
         // compiler waits for everything in flight before it uses the flat index, and at this point that is the
@@ -486,7 +473,6 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_m
       const int ks_w = ks + kWDepth < nks ? ks + kWDepth : ks + kWDepth - nks;
       if (ks + kWDepth == nks && has_next) set_wrow(nxt);
       load_step_w<QUANT, kUnits>(ks_w, wrow, du, w[P]);
-      XABE_MT(1);
       // Second barrier of the step, by hand: this wavefront's LDS stores and its activation pieces must have
       // landed, the weight loads just issued need not.  Memory operations retire in order, so "all but the last
       // kWLoadsAtLeast" covers the pieces; the count is a lower bound of the load instructions a step issues
@@ -494,7 +480,6 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_m
       order_fence();
       asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kWLoadsAtLeast) : "memory");
       order_fence();
-      XABE_MT(2);
       if (ks + 1 == nks && has_next) set_arow(buf ^ 1, nxt.rows);
       const _Float16* pa = &sA[(wm * kWaveStride + (lane & 31)) * kLdA];
       // 32-row blocks of this wavefront that hold live rows (all of them in the unrouted forms)
@@ -544,10 +529,6 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_m
           }
         }
       }
-      XABE_MT(3);
-#ifdef XABE_MFMA_TRACE
-      ++trace_step;
-#endif
     };
     if constexpr (kWDepth == 2) {
       // (at least one pair of steps, and written so: a path around the loop would count for the compiler's waits
@@ -1330,9 +1311,3 @@ int mfma_shared_expert(const xabe_moe_kernels* k, hipStream_t s, xabe_moe_buffer
 }
 
 }  // namespace xabe
-
-#ifdef XABE_MFMA_TRACE
-extern "C" int xabe_debug_read_mfma_trace(long long* out, size_t n) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(xabe::g_mfma_trace), n * sizeof(long long));
-}
-#endif

@@ -4,9 +4,6 @@
 
 #include "device_common.h"
 
-#ifndef XABE_ROUTE_TRACE
-#define XABE_ROUTE_TRACE(slot) do { } while (0)
-#endif
 
 namespace xabe {
 
@@ -124,7 +121,6 @@ __device__ __forceinline__ void route_finish(const float (&l)[PER], int num_expe
 #pragma unroll
   for (int i = 1; i < PER; ++i) m = fmaxf(m, l[i]);
   m = wave_max(m);
-  XABE_ROUTE_TRACE(1);
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int idx = i * 64 + lane;
@@ -133,7 +129,6 @@ __device__ __forceinline__ void route_finish(const float (&l)[PER], int num_expe
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  XABE_ROUTE_TRACE(2);
   // sequential sum in index order on lane 0 alone (a 16-byte LDS read that all 64 lanes aim at one
   // address is serialised lane by lane), 32 values per batch so that the reads are in flight together and
   // only the additions form the dependent chain
@@ -155,7 +150,6 @@ __device__ __forceinline__ void route_finish(const float (&l)[PER], int num_expe
     for (int i = n32; i < num_experts; ++i) sum += e_all[i];
   }
   sum = lane_bcast(sum, 0);
-  XABE_ROUTE_TRACE(3);
   // p >= +0, so the bit patterns order like the values and comparisons run on integers
   const int pj = lane < n ? __builtin_bit_cast(int, e_all[cand_i] / sum) : 0;
   const int pn = __builtin_amdgcn_ds_bpermute(((lane + 1) & 63) * 4, pj);
@@ -179,7 +173,6 @@ __device__ __forceinline__ void route_finish(const float (&l)[PER], int num_expe
     }
   }
   const float sel_p = __builtin_bit_cast(float, sel_bits);
-  XABE_ROUTE_TRACE(4);
   // sum of the selected probabilities in selection order
   float ssum = -0.0f;
   for (int k = 0; k < top_k; ++k) ssum += lane_bcast(sel_p, k);
