@@ -196,7 +196,8 @@ __device__ __forceinline__ void accum(const typename Fmt<QUANT>::Raw& r, const L
 // the same funnel loads, so the Raw it produces is bit for bit the one load_raw produces.
 //   stage_load:  issue the global loads of one step (`nbytes` live bytes starting at `chunk`, any 2-byte
 //                alignment).  The 16-byte window around them must lie inside the tensor: the host checks
-//                that the tensor starts and ends on 16-byte boundaries.
+//                that the tensor starts and ends on 16-byte boundaries, or uses stage_load_bounded for
+//                the row at the tensor's end.
 //   stage_pick:  pieces -> LDS slot -> Raw.  Slots are private to a wavefront, whose LDS operations
 //                complete in program order; the fences only keep the compiler from reordering them.
 // ---------------------------------------------------------------------------------
@@ -230,6 +231,31 @@ __device__ __forceinline__ void stage_load(const uint8_t* chunk, uint32_t nbytes
   const int lane = (int)__lane_id();
 #pragma unroll
   for (int i = 0; i < StageFmt<QUANT>::kPieces; ++i) s.p[i] = base[min(lane + 64 * i, s.last)];
+}
+
+// stage_load for a step whose last piece may reach past the tensor's end (`end`, 2-byte aligned): that piece
+// is put together from the 2-byte fields that exist, the rest of it reads as zero.
+template <int QUANT>
+__device__ __forceinline__ void stage_load_bounded(const uint8_t* chunk, uint32_t nbytes, const uint8_t* end, Staged<QUANT>& s) {
+  s.mis = (uint32_t)(reinterpret_cast<uintptr_t>(chunk) & 15u);
+  s.last = (int)((s.mis + nbytes + 15u) >> 4) - 1;
+  const stage_piece* base = reinterpret_cast<const stage_piece*>(chunk - s.mis);
+  const int lane = (int)__lane_id();
+#pragma unroll
+  for (int i = 0; i < StageFmt<QUANT>::kPieces; ++i) {
+    const stage_piece* p = base + min(lane + 64 * i, s.last);
+    if (reinterpret_cast<const uint8_t*>(p + 1) <= end) {
+      s.p[i] = *p;
+    } else {
+      const uint16_t* h = reinterpret_cast<const uint16_t*>(p);
+      const int live = (int)(end - reinterpret_cast<const uint8_t*>(p)) >> 1;
+      stage_piece v = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (j < live) v[j >> 1] |= (uint32_t)h[j] << (16 * (j & 1));
+      s.p[i] = v;
+    }
+  }
 }
 
 template <int QUANT>

@@ -29,11 +29,15 @@ struct LmHeadArgs {
   float* out;       // [*][vocab]
   int K, vocab;
   int t0, nt;       // tokens [t0, t0 + nt) are served by this launch, 1 <= nt <= TOK
+  int row_lo, row_hi;    // quantized kernels: rows [row_lo, row_hi) are served by this launch
+  const uint8_t* w_end;  // TAIL launches: one past the tensor's last byte
 };
 
 // Q8_0 / Q6_K rows.  ONE: the row is a single wavefront step (K <= 2048) and the activations are hoisted out
 // of the row loop; otherwise the contraction is walked step by step with the activations re-read per step.
-template <int QUANT, int R, int TOK, bool ONE>
+// TAIL: the launch that serves the last row of a tensor whose length is not a multiple of 16 bytes; the one
+// piece that would reach past the tensor is put together from 2-byte loads.
+template <int QUANT, int R, int TOK, bool ONE, bool TAIL = false>
 __global__ void __launch_bounds__(256) k_lm_head_quant(LmHeadArgs a) {
   using F = Fmt<QUANT>;
   using Raw = typename F::Raw;
@@ -43,7 +47,7 @@ __global__ void __launch_bounds__(256) k_lm_head_quant(LmHeadArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const size_t row_bytes = (size_t)(a.K / F::kBlockElems) * F::kBlockBytes;
   const int steps = (a.K + kStepElems - 1) / kStepElems;
-  const int groups = (a.vocab + R - 1) / R;
+  const int groups = (a.row_hi - a.row_lo + R - 1) / R;
   const int stride = (int)gridDim.x * kWavesPerWg;
   uint8_t* slots = s_slots + (size_t)wave * R * kSlot;
 
@@ -51,8 +55,10 @@ __global__ void __launch_bounds__(256) k_lm_head_quant(LmHeadArgs a) {
     const uint32_t nbytes = (uint32_t)(min(kStepElems, a.K - k * kStepElems) / F::kBlockElems) * F::kBlockBytes;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int row = min(rg * R + r, a.vocab - 1);  // a group past the last row repeats it and stores nothing
-      stage_load<QUANT>(a.w + (size_t)row * row_bytes + (size_t)k * F::kChunkBytes, nbytes, pend[r]);
+      const int row = min(a.row_lo + rg * R + r, a.row_hi - 1);  // a group past the last row repeats it and stores nothing
+      const uint8_t* chunk = a.w + (size_t)row * row_bytes + (size_t)k * F::kChunkBytes;
+      if constexpr (TAIL) stage_load_bounded<QUANT>(chunk, nbytes, a.w_end, pend[r]);
+      else stage_load<QUANT>(chunk, nbytes, pend[r]);
     }
     issue_fence();
   };
@@ -75,8 +81,8 @@ __global__ void __launch_bounds__(256) k_lm_head_quant(LmHeadArgs a) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const float tot = group_sum<64>(acc[r][t]);
-        const int row = rg * R + r;
-        if (g.lane == 0 && row < a.vocab) a.out[(size_t)(a.t0 + t) * a.vocab + row] = 1.0f * tot;
+        const int row = a.row_lo + rg * R + r;
+        if (g.lane == 0 && row < a.row_hi) a.out[(size_t)(a.t0 + t) * a.vocab + row] = 1.0f * tot;
       }
     }
   };
@@ -410,9 +416,14 @@ template <int TOK>
 static void launch_pass(const xabe_lm_head* h, hipStream_t s, int format, const LmHeadArgs& a) {
   // rows per wavefront iteration: four for one token, two once the tile's activations take the registers
   constexpr int R = TOK == 1 ? 4 : 2;
-  const int groups = (a.vocab + R - 1) / R;
+  const int groups = (a.row_hi - a.row_lo + R - 1) / R;
   const unsigned grid = (unsigned)std::max(1, std::min((groups + kWavesPerWg - 1) / kWavesPerWg, h->num_cus * 4));
   const bool one = a.K <= kStepElems;
+  if (a.w_end) {  // the last row of a tensor that ends inside a 16-byte piece: one wavefront, bounded loads
+    if (format == XABE_HEAD_Q8_0) hipLaunchKernelGGL((k_lm_head_quant<kQ8_0, R, TOK, false, true>), dim3(1), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_lm_head_quant<kQ6K, R, TOK, false, true>), dim3(1), dim3(256), 0, s, a);
+    return;
+  }
   switch (format) {
     case XABE_HEAD_Q8_0:
       if (one) hipLaunchKernelGGL((k_lm_head_quant<kQ8_0, R, TOK, true>), dim3(grid), dim3(256), 0, s, a);
@@ -462,10 +473,11 @@ int xabe_lm_head_forward(const xabe_lm_head* h, void* stream, int format, const 
   XABE_TRY(check_len("logits", g.max_tokens * g.vocab, logits_len));
   if ((reinterpret_cast<uintptr_t>(weight) & 15u) != 0 || (reinterpret_cast<uintptr_t>(hidden_states) & 15u) != 0)
     return set_error(XABE_ERR_INVALID_ARGUMENT, "LM head: the weight tensor and the hidden states must start on 16-byte boundaries");
-  // the coalesced loader reads whole 16-byte pieces: the last piece of the tensor must end inside it
+  // the coalesced loader reads whole 16-byte pieces.  A quantized tensor that ends inside one has its last row
+  // served by a launch of its own, whose loads stop at the tensor's end; the 16-byte windows of every earlier
+  // row end inside the last row.
   const bool quant = format == XABE_HEAD_Q8_0 || format == XABE_HEAD_Q6K;
-  if (quant && weight_len % 16 != 0)
-    return set_error(XABE_ERR_INVALID_ARGUMENT, "LM head: a quantized weight tensor must end on a 16-byte boundary (%zu bytes)", weight_len);
+  const bool ragged_end = quant && weight_len % 16 != 0;
   hipStream_t s = xabe::as_stream(stream);
   xabe::LmHeadArgs a;
   a.w = static_cast<const uint8_t*>(weight);
@@ -477,13 +489,19 @@ int xabe_lm_head_forward(const xabe_lm_head* h, void* stream, int format, const 
     const int tile = (int)std::min<size_t>(XABE_LM_HEAD_MAX_BATCH_TILE, tokens - base);
     a.t0 = (int)base;
     a.nt = tile;
-    switch (tile) {
-      case 1: xabe::launch_pass<1>(h, s, format, a); break;
-      case 2: xabe::launch_pass<2>(h, s, format, a); break;
-      case 3: xabe::launch_pass<3>(h, s, format, a); break;
-      default: xabe::launch_pass<4>(h, s, format, a); break;
+    for (int part = 0; part < (ragged_end ? 2 : 1); ++part) {
+      a.row_lo = part == 0 ? 0 : a.vocab - 1;
+      a.row_hi = ragged_end && part == 0 ? a.vocab - 1 : a.vocab;
+      a.w_end = part == 0 ? nullptr : a.w + weight_len;
+      if (a.row_lo >= a.row_hi) continue;  // a one-row tensor has only the bounded part
+      switch (tile) {
+        case 1: xabe::launch_pass<1>(h, s, format, a); break;
+        case 2: xabe::launch_pass<2>(h, s, format, a); break;
+        case 3: xabe::launch_pass<3>(h, s, format, a); break;
+        default: xabe::launch_pass<4>(h, s, format, a); break;
+      }
+      XABE_HIP_TRY(hipGetLastError());
     }
-    XABE_HIP_TRY(hipGetLastError());
   }
   return XABE_OK;
 }

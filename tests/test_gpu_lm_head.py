@@ -98,8 +98,7 @@ def test_formats_and_shapes(oracle, X, fmt, vocab, hidden, max_tokens, tokens):
     # lm_head_formats_differential.rs: every format, ragged vocabularies, rows of one step and of several
     fmt = getattr(X.HeadFormat, fmt)
     g = X.LmHeadGeometry(hidden, vocab, max_tokens)
-    if fmt in (X.HeadFormat.Q8_0, X.HeadFormat.Q6K) and g.weight_bytes_for(fmt) % 16:
-        pytest.skip("a quantized tensor that does not end on a 16-byte boundary is refused (see test_forward_error_paths)")
+    # Q6_K at (777, 1024) and (513, 1536) ends 8 and 12 bytes into a 16-byte piece: the last row goes through the bounded loader
     w, host = _weights(X, oracle, fmt, vocab, hidden, 32000 + vocab)
     k = X.LmHeadKernels(g)
     x = X.synth_normal_f32(32001, max_tokens * hidden, 1.0).view(max_tokens, hidden)
