@@ -141,8 +141,14 @@ constexpr int kRgRowBytes = 80;  // a 32-element bf16 row padded to 80 bytes: 16
 template <int RN>
 __global__ void __launch_bounds__(256) k_router_gemm_q8_bf16x3(RouterGemmArgs a) {
   static_assert(RN == 128 || RN == 64, "expert tile");
-  constexpr int NJ = RN / 64;    // 32-column blocks per wavefront
-  constexpr int kBPer = RN / 8;  // codes of the B tile a thread stages per step (16 or 8)
+  // wavefronts: 2 (tokens) x 2 (experts), each 32 tokens x NJ blocks of 32 experts.  (A 256-expert tile on eight
+  // wavefronts, which reads the activations once for the whole router, was measured: 92 us against 50 at 8192
+  // tokens; its 512 workgroups are too few to cover each other's loads.)
+  constexpr int kThreads = 256;
+  constexpr int WN = 2;
+  constexpr int NJ = RN / (32 * WN);
+  constexpr int kAPer = kRgM * kRgK / kThreads;  // activations a thread stages per step (8 or 4)
+  constexpr int kBPer = RN * kRgK / kThreads;    // codes of the B tile a thread stages per step (16 or 8)
   __shared__ __attribute__((aligned(16))) uint8_t sA[3 * kRgM * kRgRowBytes];
   __shared__ __attribute__((aligned(16))) uint8_t sB[RN * kRgRowBytes];
   __shared__ float sD[RN];
@@ -150,8 +156,8 @@ __global__ void __launch_bounds__(256) k_router_gemm_q8_bf16x3(RouterGemmArgs a)
   const int m0 = blockIdx.y * kRgM, n0 = blockIdx.x * RN;
   if (m0 >= valid) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int am = tid >> 2, ak = (tid & 3) * 8;
+  const int wm = wave / WN, wn = wave % WN;
+  const int am = tid / (32 / kAPer), ak = (tid % (32 / kAPer)) * kAPer;
   const float* arow = a.normed + (size_t)min(m0 + am, valid - 1) * a.H + ak;
   const int bn = tid / (32 / kBPer), bk = (tid % (32 / kBPer)) * kBPer;
   const uint8_t* brow = static_cast<const uint8_t*>(a.router) + (size_t)(n0 + bn) * (size_t)(a.H / 32) * kQ8Bytes;
@@ -162,46 +168,56 @@ __global__ void __launch_bounds__(256) k_router_gemm_q8_bf16x3(RouterGemmArgs a)
 
   const int nks_all = a.H / kRgK, ks0 = (int)blockIdx.z * (nks_all / a.splits), nks = ks0 + nks_all / a.splits;
   float* const plane = a.logits + (size_t)blockIdx.z * a.max_tokens * a.E;
-  float4 ra[2];
-  uint32_t rq[kBPer / 4 + 1];  // the aligned dwords around this thread's codes
-  uint32_t rd = 0;             // the block's scale (fp16 bits), bk == 0 threads
-  auto load_step = [&](int ks) {
-    ra[0] = reinterpret_cast<const float4*>(arow + (size_t)ks * kRgK)[0];
-    ra[1] = reinterpret_cast<const float4*>(arow + (size_t)ks * kRgK)[1];
+  // what a thread holds of one step: two steps are in flight, so that a step's loads have two steps' time to land
+  struct Held {
+    float4 ra[kAPer / 4];
+    uint32_t rq[kBPer / 4 + 1];  // the aligned dwords around this thread's codes
+    uint32_t rd;                 // the block's scale (fp16 bits), bk == 0 threads
+  };
+  auto load_step = [&](int ks, Held& h) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < kAPer / 4; ++i) h.ra[i] = reinterpret_cast<const float4*>(arow + (size_t)ks * kRgK)[i];
     // block ks of the row: d (fp16) then 32 codes; rows start on 16 bytes and a block is 34, so the codes start
     // on a dword in odd blocks and two bytes past one in even blocks (the row's block count is even: checked by
     // the host, so the dword past an even block's codes lies inside the row)
     const uint8_t* blk = brow + (size_t)ks * kQ8Bytes;
     const uint32_t* w = reinterpret_cast<const uint32_t*>(blk + (ks & 1 ? 2 : 0) + bk);
 #pragma unroll
-    for (int i = 0; i <= kBPer / 4; ++i) rq[i] = (i < kBPer / 4 || !(ks & 1)) ? w[i] : 0u;
-    if (bk == 0) rd = *reinterpret_cast<const uint16_t*>(blk);
+    for (int i = 0; i <= kBPer / 4; ++i) h.rq[i] = (i < kBPer / 4 || !(ks & 1)) ? w[i] : 0u;
+    h.rd = 0;
+    if (bk == 0) h.rd = *reinterpret_cast<const uint16_t*>(blk);
   };
-  load_step(ks0);
-  for (int ks = ks0; ks < nks; ++ks) {
+  auto step = [&](int ks, Held& h) __attribute__((always_inline)) {
+    const uint32_t (&rq)[kBPer / 4 + 1] = h.rq;
+    const uint32_t rd = h.rd;
     __syncthreads();  // the previous step's tiles have been read
     {
-      // activations: three exact bf16 pieces, eight elements = one 16-byte row segment per piece
-      const float va[8] = {ra[0].x, ra[0].y, ra[0].z, ra[0].w, ra[1].x, ra[1].y, ra[1].z, ra[1].w};
-      uint32_t p0[8], p1[8], p2[8];
+      // activations: three exact bf16 pieces, kAPer elements = one 16- or 8-byte row segment per piece
+      float va[kAPer];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kAPer / 4; ++i) {
+        va[4 * i] = h.ra[i].x; va[4 * i + 1] = h.ra[i].y; va[4 * i + 2] = h.ra[i].z; va[4 * i + 3] = h.ra[i].w;
+      }
+      uint32_t p0[kAPer], p1[kAPer], p2[kAPer];
+#pragma unroll
+      for (int i = 0; i < kAPer; ++i) {
         p0[i] = __builtin_bit_cast(uint32_t, va[i]);
         const float r1 = va[i] - __builtin_bit_cast(float, p0[i] & 0xffff0000u);
         p1[i] = __builtin_bit_cast(uint32_t, r1);
         const float r2 = r1 - __builtin_bit_cast(float, p1[i] & 0xffff0000u);
         p2[i] = __builtin_bit_cast(uint32_t, r2);
       }
-      auto pack = [](const uint32_t (&p)[8]) {
-        rg_u32x4 v;
+      typedef uint32_t piece_t __attribute__((ext_vector_type(kAPer / 2)));
+      auto pack = [&](const uint32_t (&p)[kAPer]) {
+        piece_t v;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = __builtin_amdgcn_perm(p[2 * i + 1], p[2 * i], 0x07060302u);  // two upper halves
+        for (int i = 0; i < kAPer / 2; ++i) v[i] = __builtin_amdgcn_perm(p[2 * i + 1], p[2 * i], 0x07060302u);  // two upper halves
         return v;
       };
       uint8_t* dst = sA + am * kRgRowBytes + ak * 2;
-      *reinterpret_cast<rg_u32x4*>(dst) = pack(p0);
-      *reinterpret_cast<rg_u32x4*>(dst + kRgM * kRgRowBytes) = pack(p1);
-      *reinterpret_cast<rg_u32x4*>(dst + 2 * kRgM * kRgRowBytes) = pack(p2);
+      *reinterpret_cast<piece_t*>(dst) = pack(p0);
+      *reinterpret_cast<piece_t*>(dst + kRgM * kRgRowBytes) = pack(p1);
+      *reinterpret_cast<piece_t*>(dst + 2 * kRgM * kRgRowBytes) = pack(p2);
       // codes: in even blocks they sit two bytes into the dwords that were read
       uint32_t c[kBPer / 4];
 #pragma unroll
@@ -222,18 +238,18 @@ __global__ void __launch_bounds__(256) k_router_gemm_q8_bf16x3(RouterGemmArgs a)
       if (bk == 0) sD[bn] = f16_bits_to_f32((uint16_t)rd);
     }
     __syncthreads();
-    if (ks + 1 < nks) load_step(ks + 1);  // in flight while the matrix core works
+    if (ks + 2 < nks) load_step(ks + 2, h);  // in flight during this step's and the next step's matrix work
     // operand layout of the 32x32x16 instruction: lane l supplies row (column) l % 32, k = (l / 32) * 8 .. + 8
     const uint8_t* pa = sA + (wm * 32 + (lane & 31)) * kRgRowBytes + (lane >> 5) * 16;
     bf16x8 fa[3][2];
 #pragma unroll
     for (int p = 0; p < 3; ++p)
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-        fa[p][h] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const rg_u32x4*>(pa + p * kRgM * kRgRowBytes + h * 32));
+      for (int kh = 0; kh < 2; ++kh)
+        fa[p][kh] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const rg_u32x4*>(pa + p * kRgM * kRgRowBytes + kh * 32));
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const int col = wn * (RN / 2) + j * 32 + (lane & 31);
+      const int col = wn * (RN / WN) + j * 32 + (lane & 31);
       const uint8_t* pb = sB + col * kRgRowBytes + (lane >> 5) * 16;
       const bf16x8 fb0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const rg_u32x4*>(pb));
       const bf16x8 fb1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const rg_u32x4*>(pb + 32));
@@ -247,13 +263,20 @@ __global__ void __launch_bounds__(256) k_router_gemm_q8_bf16x3(RouterGemmArgs a)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[j][v] = __builtin_fmaf(d, blk[v], acc[j][v]);
     }
+  };
+  Held h0, h1;
+  load_step(ks0, h0);
+  if (ks0 + 1 < nks) load_step(ks0 + 1, h1);
+  for (int ks = ks0; ks < nks; ks += 2) {
+    step(ks, h0);
+    if (ks + 1 < nks) step(ks + 1, h1);
   }
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
     const int t = m0 + wm * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
     if (t >= valid) continue;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) plane[(size_t)t * a.E + n0 + wn * (RN / 2) + j * 32 + (lane & 31)] = acc[j][v];
+    for (int j = 0; j < NJ; ++j) plane[(size_t)t * a.E + n0 + wn * (RN / WN) + j * 32 + (lane & 31)] = acc[j][v];
   }
 }
 
