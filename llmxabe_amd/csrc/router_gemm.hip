@@ -136,6 +136,7 @@ __global__ void __launch_bounds__(256) k_router_gemm(RouterGemmArgs a) {
 // inside a block differs), and a token's logits do not depend on its batch mates here either.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t rg_u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kRgAhead = 2;     // steps of global loads a thread keeps in flight (four: 55 us against 50 at 8192 tokens)
 constexpr int kRgRowBytes = 80;  // a 32-element bf16 row padded to 80 bytes: 16-byte reads of 32 rows hit every bank once
 
 template <int RN>
@@ -168,7 +169,7 @@ __global__ void __launch_bounds__(256) k_router_gemm_q8_bf16x3(RouterGemmArgs a)
 
   const int nks_all = a.H / kRgK, ks0 = (int)blockIdx.z * (nks_all / a.splits), nks = ks0 + nks_all / a.splits;
   float* const plane = a.logits + (size_t)blockIdx.z * a.max_tokens * a.E;
-  // what a thread holds of one step: two steps are in flight, so that a step's loads have two steps' time to land
+  // what a thread holds of one step: kRgAhead steps are in flight, so that a step's loads have that many steps' time to land
   struct Held {
     float4 ra[kAPer / 4];
     uint32_t rq[kBPer / 4 + 1];  // the aligned dwords around this thread's codes
@@ -238,7 +239,7 @@ __global__ void __launch_bounds__(256) k_router_gemm_q8_bf16x3(RouterGemmArgs a)
       if (bk == 0) sD[bn] = f16_bits_to_f32((uint16_t)rd);
     }
     __syncthreads();
-    if (ks + 2 < nks) load_step(ks + 2, h);  // in flight during this step's and the next step's matrix work
+    if (ks + kRgAhead < nks) load_step(ks + kRgAhead, h);  // in flight during the next kRgAhead steps' matrix work
     // operand layout of the 32x32x16 instruction: lane l supplies row (column) l % 32, k = (l / 32) * 8 .. + 8
     const uint8_t* pa = sA + (wm * 32 + (lane & 31)) * kRgRowBytes + (lane >> 5) * 16;
     bf16x8 fa[3][2];
@@ -264,12 +265,14 @@ __global__ void __launch_bounds__(256) k_router_gemm_q8_bf16x3(RouterGemmArgs a)
       for (int v = 0; v < 16; ++v) acc[j][v] = __builtin_fmaf(d, blk[v], acc[j][v]);
     }
   };
-  Held h0, h1;
-  load_step(ks0, h0);
-  if (ks0 + 1 < nks) load_step(ks0 + 1, h1);
-  for (int ks = ks0; ks < nks; ks += 2) {
-    step(ks, h0);
-    if (ks + 1 < nks) step(ks + 1, h1);
+  Held held[kRgAhead];
+#pragma unroll
+  for (int d = 0; d < kRgAhead; ++d)
+    if (ks0 + d < nks) load_step(ks0 + d, held[d]);
+  for (int ks = ks0; ks < nks; ks += kRgAhead) {
+#pragma unroll
+    for (int d = 0; d < kRgAhead; ++d)
+      if (ks + d < nks) step(ks + d, held[d]);
   }
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
