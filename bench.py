@@ -509,8 +509,9 @@ def stack_workload(args, workload, T, L) -> dict:
     """L independently seeded MoE layers resident at once, one pass of T tokens through all of them per step:
     layer l's l_out (residual + block output) is layer l + 1's input, with the RMSNorm between them either as the
     next block's first step (`value`: the reference-shaped calls) or folded into the launch that finishes l_out (the
-    `seam` object: xabe_moe_block_forward_seam, same bits).  Ping-pong activation buffers, eager launches, HIP events on
-    the launch stream."""
+    `seam` object: xabe_moe_block_forward_seam, same bits).  Ping-pong activation buffers, HIP events on the launch
+    stream; at decode widths the whole pass is one hipGraph (as a decode engine would replay it: eager launches of
+    three ~10 us kernels per layer are bound by the host), wider passes are launched eagerly."""
     import numpy as np
     import torch
 
@@ -539,16 +540,25 @@ def stack_workload(args, workload, T, L) -> dict:
         return cur
 
     reps_w, reps = max(1, min(args.warmup, 4)), max(2, min(args.steps, 16 if T < 512 else 4))
+    use_graph = T <= 32 and not args.no_graph
     times, outs = {}, {}
     with torch.cuda.stream(stream):
         for seam in (False, True):
             for _ in range(reps_w):
-                one_pass(seam)
+                out = one_pass(seam)
             stream.synchronize()
+            run = lambda: one_pass(seam)  # noqa: E731
+            if use_graph:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=stream):
+                    one_pass(seam)
+                graph.replay()
+                stream.synchronize()
+                run = graph.replay
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
             for _ in range(reps):
-                out = one_pass(seam)
+                run()
             e1.record(stream)
             e1.synchronize()
             times[seam] = e0.elapsed_time(e1) / reps
@@ -581,7 +591,7 @@ def stack_workload(args, workload, T, L) -> dict:
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands, f32 accumulate" if mfma else "f32", "data": "synthetic",
         "config": {"workload": "moe_stack_" + workload, "layers": L, "tokens": T, "num_experts": 256, "top_k": 8,
                    "hidden": 2048, "intermediate": 512, "expert_quant": "Q6_K", "shared_and_router_quant": "Q8_0",
-                   "resident_weight_bytes": weight_bytes, "launch": "eager", "us_per_layer": ms * 1e3 / L,
+                   "resident_weight_bytes": weight_bytes, "launch": "hipGraph" if use_graph else "eager", "us_per_layer": ms * 1e3 / L,
                    "output_finite": finite},
         "seam": {"what": "the same pass with every layer boundary's RMSNorm folded into the launch that finishes l_out "
                          "(xabe_moe_block_forward_seam; no ffn_out / routed read-back tensors)",
