@@ -161,8 +161,10 @@ int long_rows_configure() {
                         reinterpret_cast<const void*>(k_shared_long_rows<kQ8_0, 2, 2, 4, false, true>)};
   for (const void* f : fns)
     XABE_HIP_TRY(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLongRowsLdsMax));
-  const void* staged[6] = {reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 2, 2, false>),
+  const void* staged[8] = {reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 2, 2, false>),
                            reinterpret_cast<const void*>(k_long_rows_staged<kQ8_0, 2, 2, false>),
+                           reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 2, 1, false>),
+                           reinterpret_cast<const void*>(k_long_rows_staged<kQ8_0, 2, 1, false>),
                            reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 1, 4, false>),
                            reinterpret_cast<const void*>(k_long_rows_staged<kQ8_0, 1, 4, false>),
                            reinterpret_cast<const void*>(k_long_rows_staged<kQ6K, 1, 4, true>),
@@ -212,9 +214,27 @@ bool launch_long_rows(const xabe_moe_kernels* k, int quant, int nm, const LongRo
     // projection: 5120 rows, 160 against 256 groups): ten wavefronts of two rows
     const bool ten = nm == 1 && a.n_rows % 20 == 0 && groups8 < (unsigned)k->num_cus && (unsigned)(a.n_rows / 20) >= groups8 * 3 / 2;
     const dim3 grid10(std::min<unsigned>((unsigned)(a.n_rows / 20), (unsigned)k->num_cus), pass8), block10(640);
+    // gate/up whose groups do not divide evenly over the CUs (17408 row pairs: 1088 groups of 16 on 256 CUs, a fifth
+    // round for a quarter of them): whole rounds in the main launch, the left-over rows as half-size groups (one row
+    // pair per wavefront) spread over twice as many CUs in a second launch
+    LongRowArgs la_main = la, la_rest = la;
+    unsigned rest_groups = 0;
+    if (nm == 2 && groups8 > (unsigned)k->num_cus && groups8 % (unsigned)k->num_cus != 0 &&
+        2 * (groups8 % (unsigned)k->num_cus) <= (unsigned)k->num_cus) {
+      const unsigned whole = groups8 / (unsigned)k->num_cus * (unsigned)k->num_cus;
+      la_main.row_begin = 0;
+      la_main.row_end = (int)(whole * 8 * r);
+      la_rest.row_begin = la_main.row_end;
+      la_rest.row_end = a.n_rows;
+      rest_groups = (groups8 - whole) * 2;
+    }
 #define XABE_STAGED(Q)                                                                                                          \
   do {                                                                                                                          \
-    if (nm == 2) hipLaunchKernelGGL((k_long_rows_staged<Q, 2, 2, false>), grid8, block8, kStagedLdsBytes, s, la);               \
+    if (nm == 2) {                                                                                                              \
+      hipLaunchKernelGGL((k_long_rows_staged<Q, 2, 2, false>), grid8, block8, kStagedLdsBytes, s, la_main);                     \
+      if (rest_groups)                                                                                                          \
+        hipLaunchKernelGGL((k_long_rows_staged<Q, 2, 1, false>), dim3(rest_groups, pass8), block8, kStagedLdsBytes, s, la_rest); \
+    }                                                                                                                           \
     else if (ten && resid) hipLaunchKernelGGL((k_long_rows_staged<Q, 1, 2, true, 10>), grid10, block10, kStagedLdsBytes, s, la); \
     else if (ten) hipLaunchKernelGGL((k_long_rows_staged<Q, 1, 2, false, 10>), grid10, block10, kStagedLdsBytes, s, la);        \
     else if (resid) hipLaunchKernelGGL((k_long_rows_staged<Q, 1, 4, true>), grid8, block8, kStagedLdsBytes, s, la);             \

@@ -642,6 +642,7 @@ struct LongRowArgs {
   ExpertArgs m;
   const float* residual;  // RESID
   float* l_out;           // RESID
+  int row_begin, row_end;  // k_long_rows_staged: the launch serves rows [row_begin, row_end); row_end 0 = all of them
 };
 
 //   XLDS:   the pass's activation rows are copied into LDS once per workgroup and every step reads its 32
@@ -806,7 +807,9 @@ __global__ void __launch_bounds__(64 * WAVES, WAVES > 8 ? 3 : 2) k_long_rows_sta
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const size_t row_bytes = (size_t)(a.K / F::kBlockElems) * F::kBlockBytes;
   const int steps = (a.K + kStepElems - 1) / kStepElems;
-  const int n_groups = a.n_rows / (WAVES * R);
+  // groups of WAVES x R rows; this launch's range starts at group g0 (the host cuts ranges at group boundaries)
+  const int g0 = la.row_begin / (WAVES * R);
+  const int n_groups = (la.row_end ? la.row_end : a.n_rows) / (WAVES * R) - g0;
   if ((int)blockIdx.x >= n_groups) return;
   const int n_mine = (n_groups - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
   const int total = n_mine * steps;
@@ -866,7 +869,7 @@ __global__ void __launch_bounds__(64 * WAVES, WAVES > 8 ? 3 : 2) k_long_rows_sta
 
   Raw raw_next[RW];
   stage(0, 0);
-  load_rows((int)blockIdx.x, 0, raw_next);
+  load_rows(g0 + (int)blockIdx.x, 0, raw_next);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   finish_stage(0, 0);
@@ -877,7 +880,7 @@ __global__ void __launch_bounds__(64 * WAVES, WAVES > 8 ? 3 : 2) k_long_rows_sta
   for (int rw = 0; rw < RW; ++rw)
 #pragma unroll
     for (int t = 0; t < TOK; ++t) tot[rw][t] = 0.0f;
-  int grp = (int)blockIdx.x, s = 0;
+  int grp = g0 + (int)blockIdx.x, s = 0;
 #pragma unroll 1
   for (int i = 0; i < total; ++i) {
     const int b = i & 1;

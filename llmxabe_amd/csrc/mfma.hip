@@ -611,8 +611,7 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_m
 // never ahead (8192 tokens: gate/up 461 against 421 us, down 333 against 308), so it is not the default.  It is kept
 // because it is the measured answer to "would wavefronts that only dequantise beside wavefronts that only multiply
 // overlap the two kinds of work": they do not.  On a SIMD the producers' vector instructions and the consumers'
-// matrix instructions take turns (per 64-element step and SIMD: 1024 cycles of matrix instructions + 1144 of vector
-// instructions of work, 1320 ns = 3170 cycles of wall time; either kind alone, the other removed, still takes ~2600),
+// matrix instructions take turns,
 // so what decides the time is the sum of the two per token row, and that sum is smallest for the tallest token tile
 // (one dequantisation per expert), whose accumulators only fit a few fat wavefronts: k_mfma_expert's 384-row form.
 //
