@@ -42,7 +42,7 @@ def test_wrappers_call_declared_functions_with_the_declared_arity():
         arity[m.group(1)] = 0 if not args else len(args.split(", "))
     consts = set(re.findall(r"pub const (XABE_\w+):", ffi))
     calls = 0
-    for name in ("moe.rs", "block.rs", "layer_ops.rs"):
+    for name in ("moe.rs", "block.rs", "layer_ops.rs", "dense.rs", "lm_head.rs", "weights.rs"):
         src = open(os.path.join(CRATE, "src", name)).read()
         for m in re.finditer(r"ffi::(xabe_\w+)\s*\(", src):
             fn = m.group(1)

@@ -136,6 +136,9 @@ impl MoeBlockHandle {
     pub fn geometry(&self) -> MoeGeometry {
         self.geometry
     }
+    pub(crate) fn raw_mut(&mut self) -> *mut ffi::xabe_moe_block {
+        self.raw
+    }
     /// block/moe.rs:1081-1089: outside graph capture.
     pub fn publish_tokens(&mut self, stream: &Arc<HipStream>, tokens: usize) -> Result<(), MoeError> {
         check(unsafe { ffi::xabe_moe_block_publish_tokens(self.raw, stream.raw(), tokens) })
@@ -213,4 +216,34 @@ impl Drop for MoeBlockHandle {
     fn drop(&mut self) {
         unsafe { ffi::xabe_moe_block_free(self.raw) }
     }
+}
+
+/// `MoeBlockHandle::forward` at decode widths for callers that cannot allocate device memory (no counterpart in the
+/// reference): no handle, the block's working set sits in a device array the library holds statically on each GPU.
+/// Limit: `max_tokens` <= 32, hidden <= 2048, intermediate <= 512, <= 512 experts, top-k <= 8; calls that overlap on
+/// one GPU race; the first call on a device must not be under stream capture.
+#[allow(clippy::too_many_arguments)]
+pub fn block_forward_noalloc(
+    stream: &Arc<HipStream>,
+    geometry: &MoeGeometry,
+    eps: f32,
+    w: &MoeLayerWeights<'_>,
+    residual: &HipSlice<f32>,
+    tokens: usize,
+    ffn_out: &mut HipSlice<f32>,
+    l_out: &mut HipSlice<f32>,
+) -> Result<(), MoeError> {
+    let g = ffi::xabe_moe_geometry {
+        num_experts: geometry.num_experts,
+        experts_per_token: geometry.experts_per_token,
+        hidden: geometry.hidden,
+        intermediate: geometry.intermediate,
+        block_size: geometry.block_size,
+        max_tokens: geometry.max_tokens,
+    };
+    let cw = w.raw();
+    check(unsafe {
+        ffi::xabe_moe_block_forward_noalloc(&g, eps, stream.raw(), &cw, residual.as_ptr(), residual.len(), tokens, std::ptr::null(),
+                                            ffn_out.as_mut_ptr(), ffn_out.len(), l_out.as_mut_ptr(), l_out.len())
+    })
 }

@@ -13,12 +13,18 @@
 //! * [`layer_ops`] `LayerOpsKernels::rms_norm`
 //! * [`block`]   what `block/moe.rs` compiled for itself through NVRTC (router logits, gate-and-combine) as library
 //!               calls, and the whole-block entry points (`MoeBlockHandle`: three launches at decode widths, the
-//!               seam to the next layer's RMSNorm)
+//!               seam to the next layer's RMSNorm; `block_forward_noalloc`)
+//! * [`dense`]   `DenseFfnBlock`, `DenseFfnLayerWeights`
+//! * [`lm_head`] `LmHeadKernels`, `LmHeadGeometry`, `HeadTensor`, `HeadFormat`
+//! * [`weights`] `GgufFile` and the upload of a layer's tensors (`UploadedMoeLayer`, `UploadedDenseFfnLayer`)
 pub mod block;
+pub mod dense;
 pub mod driver;
 pub mod ffi;
 pub mod layer_ops;
+pub mod lm_head;
 pub mod moe;
+pub mod weights;
 
 pub use driver::{DriverError, HipContext, HipSlice, HipStream};
 pub use moe::{
