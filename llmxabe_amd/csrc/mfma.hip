@@ -67,6 +67,12 @@ struct MfmaArgs {
   int top_k;
 };
 
+// SwiGLU's gate in the matrix-core regime: x / (1 + e^-x) from the hardware's exp2 and reciprocal (a few ulp of
+// fp32; the product is rounded to fp16 right after, 2^-11).  The fp32 regimes keep silu_f, whose bits they pin.
+__device__ __forceinline__ float silu_fast(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * x));
+}
+
 __device__ __forceinline__ int w_swizzle(int row) {
   return (row & 8) | ((row & 1) << 2) | ((row >> 1) & 3);
 }
@@ -575,7 +581,7 @@ __global__ void __launch_bounds__(TBM == 384 ? 512 : 256, TBM == 64 ? 3 : 2) k_m
           if (NM == 2) {
             const int col = cur.nt * 64 + wn * 32 + (lane & 31);
             const float g = acc[M0 + mi][0][v] * kWScaleInv, u = acc[M0 + mi][1][v] * kWScaleInv;
-            static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_f(g) * u);
+            static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_fast(g) * u);
           } else {
             const float sc = scs[mi][v];
 #pragma unroll
@@ -986,7 +992,7 @@ __global__ void __launch_bounds__(1024, 4) k_mfma_pc(MfmaArgs a) {
           // column blocks 0 and 1: gate and the matching up columns
           const int col = cur.nt * (kPR / 2) + wq * 32 + (lane & 31);
           const float g = acc[mi][0][v] * kWScaleInv, u = acc[mi][1][v] * kWScaleInv;
-          static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_f(g) * u);
+          static_cast<_Float16*>(a.out)[(size_t)orow * a.n_rows + col] = (_Float16)(silu_fast(g) * u);
         } else {
 #pragma unroll
           for (int ni = 0; ni < 2; ++ni) {
